@@ -39,6 +39,8 @@ _LAZY: dict[str, str] = {
     "fokulorn": "rapid_llm_amd.models.fokulorn",
     "Sikevik": "rapid_llm_amd.models.sikevik",
     "sikevik": "rapid_llm_amd.models.sikevik",
+    "Miborax": "rapid_llm_amd.models.miborax",
+    "miborax": "rapid_llm_amd.models.miborax",
 }
 
 

@@ -5,7 +5,8 @@
 // [max(0, pos - window + 1), pos] of that request through its block table
 // (window 0: all keys), which were written before this kernel runs.  With a window, the first
 // keep_first keys of the request are read as well; a value head has dv channels, which need not
-// be d; with `sink` the softmax's denominator has one more term, exp(0): a key without a value.
+// be d; with `sink` the softmax's denominator has one more term, exp(0) or, with `sink_values`,
+// exp of a number per query head: a key without a value.
 //
 // Scores (q . k) / sqrt(d) (rapid_llm/modules/attention.py:62), online softmax over tiles
 // of 256 keys in ascending order (rapid_llm/kernels/ops/attention/flashattention2_nopad.py:
@@ -20,7 +21,7 @@ __global__ __launch_bounds__(ATT_THREADS) void attention_generic_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     T* __restrict__ out, const int* __restrict__ positions, const int* __restrict__ token_slot,
     const int* __restrict__ block_table, int table_stride, int page_size, int nq, int nkv, int d,
-    int window, float scale, int dv, int keep_first, int sink) {
+    int window, float scale, int dv, int keep_first, int sink, const float* __restrict__ sink_values) {
     __shared__ float qs[256];
     __shared__ float ps[ATT_THREADS];
     __shared__ int key_page[ATT_THREADS];  // page * nkv + kv head of each key of the tile
@@ -76,7 +77,15 @@ __global__ __launch_bounds__(ATT_THREADS) void attention_generic_kernel(
         }
         __syncthreads();  // ps / key_* are rewritten by the next tile
     }
-    if (sink) l += expf(-m);
+    if (sink) {
+        // a key without a value: its score is 0, or a number of the head (never scaled); it may
+        // lie above every real score, so the state is brought to the larger maximum first
+        const float s0 = sink_values ? sink_values[h] : 0.f;
+        const float m_new = fmaxf(m, s0);
+        const float fa = expf(m - m_new);
+        l = l * fa + expf(s0 - m_new);
+        acc *= fa;
+    }
     if (tid < dv) out[((size_t)t * nq + h) * dv + tid] = from_float<T>(acc / l);
 }
 
@@ -84,7 +93,8 @@ extern "C" int rl_attention_generic(const void* q, const void* k_cache, const vo
                                     void* out, const int* positions, const int* token_slot,
                                     const int* block_table, int table_stride, int page_size,
                                     int tokens, int nq, int nkv, int d, int window, float scale,
-                                    int dv, int keep_first, int sink, int act_type, hipStream_t stream) {
+                                    int dv, int keep_first, int sink, const float* sink_values, int act_type,
+                                    hipStream_t stream) {
     if (tokens <= 0) return RL_OK;
     if (d < 1 || d > 256 || dv < 1 || dv > 256 || keep_first < 0 || nkv < 1 || nq % nkv || page_size < 1 ||
         nq > 65535)
@@ -94,12 +104,12 @@ extern "C" int rl_attention_generic(const void* q, const void* k_cache, const vo
         hipLaunchKernelGGL(attention_generic_kernel<float>, grid, block, 0, stream,
                            (const float*)q, (const float*)k_cache, (const float*)v_cache,
                            (float*)out, positions, token_slot, block_table, table_stride,
-                           page_size, nq, nkv, d, window, scale, dv, keep_first, sink);
+                           page_size, nq, nkv, d, window, scale, dv, keep_first, sink, sink_values);
     else if (act_type == RL_BF16)
         hipLaunchKernelGGL(attention_generic_kernel<bf16_t>, grid, block, 0, stream,
                            (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
                            (bf16_t*)out, positions, token_slot, block_table, table_stride,
-                           page_size, nq, nkv, d, window, scale, dv, keep_first, sink);
+                           page_size, nq, nkv, d, window, scale, dv, keep_first, sink, sink_values);
     else
         return RL_ERR_ARG;
     return rl_launch_status();

@@ -137,7 +137,7 @@ __global__ __launch_bounds__(AW* RL_WAVE) void attn_tile_kernel(
     T* __restrict__ out, const int* __restrict__ tile_info, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
     int page_size, int nq, int nkv, int window, int keep_first, int sink, float scale,
-    float* __restrict__ part, int nsplit) {
+    float* __restrict__ part, int nsplit, const float* __restrict__ sink_values) {
     typedef typename Quad<T>::type quad;
     if constexpr (sizeof(T) == 2) scale *= 1.4426950408889634f;  // scores in units of log2
     const int tile = blockIdx.x;
@@ -433,8 +433,23 @@ __global__ __launch_bounds__(AW* RL_WAVE) void attn_tile_kernel(
             }
             continue;
         }
-        // the key of score 0 that has no value: exp(0 - m) more in the denominator
-        if (sink) l[r] += fexp<T>(-m[r]);
+        // the key of score 0 that has no value: exp(0 - m) more in the denominator; with
+        // `sink_values` its score is a number of the row's head (not scaled), which may lie
+        // above every real score: the state is brought to the larger maximum first
+        if (sink) {
+            float s0 = 0.f;
+            if (sink_values) {
+                s0 = sink_values[head[r]];
+                if constexpr (sizeof(T) == 2) s0 *= 1.4426950408889634f;
+            }
+            const float m_new = fmaxf(m[r], s0);
+            const float fa = fexp<T>(m[r] - m_new);
+            l[r] = l[r] * fa + fexp<T>(s0 - m_new);
+#pragma unroll
+            for (int b = 0; b < VB; ++b)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[r][b][i] *= fa;
+        }
         // acc[r][b][i] is channel 16b + 4g + i of the lane's row
         T* orow = out + ((size_t)(at + tok[r]) * nq + head[r]) * DV + 4 * g;
         const float inv = 1.f / l[r];
@@ -449,17 +464,21 @@ __global__ __launch_bounds__(AW* RL_WAVE) void attn_tile_kernel(
 // run), add the sink's term and write the row.  One wave a row, a lane a channel (and more).
 __global__ __launch_bounds__(256) void attn_tile_merge_kernel(const float* __restrict__ part,
                                                               bf16_t* __restrict__ out, int rows, int nsplit,
-                                                              int sink) {
+                                                              int sink, const float* __restrict__ sink_values,
+                                                              int nq) {
     const int row = blockIdx.x * 4 + threadIdx.x / RL_WAVE;
     const int lane = threadIdx.x & (RL_WAVE - 1);
     if (row >= rows) return;
     const float* p = part + (size_t)row * nsplit * (DV + 2);
     float top = -INFINITY;
     for (int s = 0; s < nsplit; ++s) top = fmaxf(top, p[s * (DV + 2) + DV]);
+    // the sink's score: 0, or a number of the row's head (rows are (token, head) pairs)
+    const float s0 = (sink && sink_values) ? sink_values[row % nq] * 1.4426950408889634f : 0.f;
+    if (sink) top = fmaxf(top, s0);
     float den = 0.f;
     for (int s = 0; s < nsplit; ++s)
         den += __builtin_amdgcn_exp2f(p[s * (DV + 2) + DV] - top) * p[s * (DV + 2) + DV + 1];
-    if (sink) den += __builtin_amdgcn_exp2f(-top);
+    if (sink) den += __builtin_amdgcn_exp2f(s0 - top);
     for (int c = lane; c < DV; c += RL_WAVE) {
         float sum = 0.f;
         for (int s = 0; s < nsplit; ++s)
@@ -486,7 +505,7 @@ extern "C" int rl_attn_tile(const void* q, const void* k_cache, const void* v_ca
                             const int* token_slot, const int* block_table, int table_stride,
                             int page_size, int nq, int nkv, int window, int keep_first, int sink,
                             float scale, int nsplit, float* part, int tokens, int tile_rows, int act_type,
-                            hipStream_t stream) {
+                            const float* sink_values, hipStream_t stream) {
     if (num_tiles <= 0) return RL_OK;
     if (nkv < 1 || nq % nkv || page_size < 4 || page_size % 4 || nkv > 65535 || window < 0 || keep_first < 0)
         return RL_ERR_ARG;
@@ -499,7 +518,7 @@ extern "C" int rl_attn_tile(const void* q, const void* k_cache, const void* v_ca
     if (act_type == RL_BF16 && tile_rows == 16 * PB && PB > 1) {
         if (nsplit != 1) return RL_ERR_ARG;
         hipLaunchKernelGGL((tileattn::attn_tile_kernel<bf16_t, AW, PB>), grid, block, 0, stream, RL_TILE_ARGS(bf16_t),
-                           nullptr, 1);
+                           nullptr, 1, sink_values);
         return rl_launch_status();
     }
     if (tile_rows != 16) return RL_ERR_ARG;
@@ -509,18 +528,18 @@ extern "C" int rl_attn_tile(const void* q, const void* k_cache, const void* v_ca
     if (nsplit > 1) {
         if (act_type != RL_BF16 || !part || nsplit > 64 || tokens < 1) return RL_ERR_ARG;
         hipLaunchKernelGGL((tileattn::attn_tile_kernel<bf16_t, AW, 1>), dim3(num_tiles, nkv, nsplit), block, 0, stream,
-                           RL_TILE_ARGS(bf16_t), part, nsplit);
+                           RL_TILE_ARGS(bf16_t), part, nsplit, sink_values);
         const int rows = tokens * nq;
         hipLaunchKernelGGL(tileattn::attn_tile_merge_kernel, dim3((rows + 3) / 4), dim3(256), 0, stream, part,
-                           (bf16_t*)out, rows, nsplit, sink);
+                           (bf16_t*)out, rows, nsplit, sink, sink_values, nq);
         return rl_launch_status();
     }
     if (act_type == RL_F32)
         hipLaunchKernelGGL((tileattn::attn_tile_kernel<float, AW, 1>), grid, block, 0, stream, RL_TILE_ARGS(float),
-                           nullptr, 1);
+                           nullptr, 1, sink_values);
     else if (act_type == RL_BF16)
         hipLaunchKernelGGL((tileattn::attn_tile_kernel<bf16_t, AW, 1>), grid, block, 0, stream, RL_TILE_ARGS(bf16_t),
-                           nullptr, 1);
+                           nullptr, 1, sink_values);
     else
         return RL_ERR_ARG;
 #undef RL_TILE_ARGS

@@ -513,10 +513,13 @@ extern "C" int rl_add_rmsnorm_parts(float* residual, const float* parts, int npa
 // limit <= 0: SwiGLU, silu(g) * u (rapid_llm/kernels/ops/activation/swiglu.py:91-121).
 // limit > 0: the clamped variant, g' = min(g, limit), u' = clamp(u, -limit, limit),
 // g' * sigmoid(alpha * g') * (u' + 1).
+// With `route` (float32 [tokens, experts]) the first experts * ff hidden units of a row are those
+// of `experts` experts side by side, and expert e's are multiplied by route[t, e].
 // --------------------------------------------------------------------------- //
 template <typename T>
 __global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inter,
-                              size_t total, float limit, float alpha) {
+                              size_t total, float limit, float alpha, const float* __restrict__ route,
+                              int experts, int ff) {
     size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t step = (size_t)gridDim.x * blockDim.x;
     for (; idx < total; idx += step) {
@@ -525,7 +528,9 @@ __global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out
         const T* row = gate_up + t * 2 * (size_t)inter;
         const float g = to_float(row[j]);
         const float u = to_float(row[inter + j]);
-        out[idx] = from_float<T>(glu_act(g, u, limit, alpha));
+        float v = glu_act(g, u, limit, alpha);
+        if (route && j < experts * ff) v *= route[t * experts + j / ff];
+        out[idx] = from_float<T>(v);
     }
 }
 
@@ -537,7 +542,8 @@ struct alignas(sizeof(T) * 8) Vec8 {
 
 template <typename T>
 __global__ void swiglu_vec_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inter,
-                                  size_t total_vec, float limit, float alpha) {
+                                  size_t total_vec, float limit, float alpha, const float* __restrict__ route,
+                                  int experts, int ff) {
     size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t step = (size_t)gridDim.x * blockDim.x;
     const int per_row = inter >> 3;
@@ -547,10 +553,12 @@ __global__ void swiglu_vec_kernel(const T* __restrict__ gate_up, T* __restrict__
         const T* row = gate_up + t * 2 * (size_t)inter;
         const Vec8<T> g = *reinterpret_cast<const Vec8<T>*>(row + j);
         const Vec8<T> u = *reinterpret_cast<const Vec8<T>*>(row + inter + j);
+        // (with a route, an expert's hidden units are a multiple of 8: one factor a group)
+        const float factor = (route && j < experts * ff) ? route[t * experts + j / ff] : 1.f;
         Vec8<T> y;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            y.v[i] = from_float<T>(glu_act(to_float(g.v[i]), to_float(u.v[i]), limit, alpha));
+            y.v[i] = from_float<T>(glu_act(to_float(g.v[i]), to_float(u.v[i]), limit, alpha) * factor);
         }
         *reinterpret_cast<Vec8<T>*>(out + t * (size_t)inter + j) = y;
     }
@@ -558,29 +566,31 @@ __global__ void swiglu_vec_kernel(const T* __restrict__ gate_up, T* __restrict__
 
 template <typename T>
 static void launch_swiglu(const T* gate_up, T* out, int tokens, int inter, float limit, float alpha,
-                          hipStream_t stream) {
-    if (inter % 8 == 0) {
+                          const float* route, int experts, int ff, hipStream_t stream) {
+    if (inter % 8 == 0 && (!route || ff % 8 == 0)) {
         const size_t total = (size_t)tokens * (inter / 8);
         size_t blocks = (total + 255) / 256;
         if (blocks > 65536) blocks = 65536;
         hipLaunchKernelGGL(swiglu_vec_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream,
-                           gate_up, out, inter, total, limit, alpha);
+                           gate_up, out, inter, total, limit, alpha, route, experts, ff);
         return;
     }
     const size_t total = (size_t)tokens * inter;
     size_t blocks = (total + 255) / 256;
     if (blocks > 65536) blocks = 65536;
     hipLaunchKernelGGL(swiglu_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, gate_up, out,
-                       inter, total, limit, alpha);
+                       inter, total, limit, alpha, route, experts, ff);
 }
 
 extern "C" int rl_swiglu(const void* gate_up, void* out, int tokens, int inter, int act_type,
-                         float limit, float alpha, hipStream_t stream) {
+                         float limit, float alpha, const float* route, int experts, int ff, hipStream_t stream) {
     if (tokens <= 0) return RL_OK;
+    if (route && (experts < 1 || ff < 1 || (long)experts * ff > inter)) return RL_ERR_ARG;
     if (act_type == RL_F32)
-        launch_swiglu<float>((const float*)gate_up, (float*)out, tokens, inter, limit, alpha, stream);
+        launch_swiglu<float>((const float*)gate_up, (float*)out, tokens, inter, limit, alpha, route, experts, ff, stream);
     else if (act_type == RL_BF16)
-        launch_swiglu<bf16_t>((const bf16_t*)gate_up, (bf16_t*)out, tokens, inter, limit, alpha, stream);
+        launch_swiglu<bf16_t>((const bf16_t*)gate_up, (bf16_t*)out, tokens, inter, limit, alpha, route, experts,
+                              ff, stream);
     else
         return RL_ERR_ARG;
     return rl_launch_status();
@@ -724,11 +734,12 @@ extern "C" int rl_route(float* z, int tokens, int experts, int top, float scale,
 // The router's product and the weights in one kernel: a wave takes a token, computes
 // z_e = w[e] . x[t] in float32 for every expert (lanes stride the row, their sums are folded by
 // the wave: one order of summation per token whatever else is in the step), and its first
-// lane turns the logits into weights.  x may be bfloat16 or float32; w is float32.
+// lane turns the logits into weights.  x may be bfloat16 or float32; w is float32; `bias`
+// (optional, float32, one number an expert) is added to the logits.
 template <typename T>
 __global__ __launch_bounds__(256) void router_kernel(const T* __restrict__ x, const float* __restrict__ w,
                                                      float* __restrict__ route, int tokens, int k, int experts,
-                                                     int top, float scale) {
+                                                     int top, float scale, const float* __restrict__ bias) {
     extern __shared__ float s_logits[];  // [4][experts]
     const int lane = threadIdx.x & (RL_WAVE - 1);
     const int wave = threadIdx.x / RL_WAVE;
@@ -769,24 +780,24 @@ __global__ __launch_bounds__(256) void router_kernel(const T* __restrict__ x, co
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const float sum = wave_sum(acc[j]);
-            if (lane == 0 && j < ne) z[e0 + j] = sum;
+            if (lane == 0 && j < ne) z[e0 + j] = bias ? sum + bias[e0 + j] : sum;
         }
     }
     if (lane == 0) route_row(z, route + (size_t)t * experts, experts, top, scale);
 }
 
 extern "C" int rl_router(const void* x, const float* w, float* route, int tokens, int k, int experts, int top,
-                         float scale, int act_type, hipStream_t stream) {
+                         float scale, const float* bias, int act_type, hipStream_t stream) {
     if (tokens <= 0) return RL_OK;
     if (k < 1 || experts < 1 || experts > ROUTE_MAX_EXPERTS || top < 1 || top > experts) return RL_ERR_ARG;
     dim3 grid((tokens + 3) / 4), block(256);
     const size_t lds = (size_t)4 * experts * sizeof(float);
     if (act_type == RL_F32)
         hipLaunchKernelGGL(router_kernel<float>, grid, block, lds, stream, (const float*)x, w, route, tokens, k,
-                           experts, top, scale);
+                           experts, top, scale, bias);
     else if (act_type == RL_BF16)
         hipLaunchKernelGGL(router_kernel<bf16_t>, grid, block, lds, stream, (const bf16_t*)x, w, route, tokens, k,
-                           experts, top, scale);
+                           experts, top, scale, bias);
     else
         return RL_ERR_ARG;
     return rl_launch_status();

@@ -43,6 +43,7 @@ CORE_SOURCES = (
     "sampling.hip",
     "gemm_bf16.hip",
     "gemm_rows.hip",
+    "latent.hip",
 )
 ATTENTION_SOURCES = ("attention_mfma.hip", "attention_f32.hip")
 MLSTM_SOURCES = ("mlstm.hip",)

@@ -297,10 +297,11 @@ def route(logits: torch.Tensor, top: int, scale: float) -> None:
     _ok(core().rl_route(_p(logits), tokens, experts, top, ctypes.c_float(scale), _stream()), "rl_route")
 
 
-def router(x: torch.Tensor, w: torch.Tensor, top: int, scale: float) -> torch.Tensor:
+def router(x: torch.Tensor, w: torch.Tensor, top: int, scale: float, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The experts' weights ``[tokens, experts]`` (float32) of rows ``x`` under the float32 router
-    matrix ``w [experts, k]``: the product in float32, softmax over all experts, the ``top``
-    largest scores over their sum (+ 1e-20) times ``scale``, 0 elsewhere.  One kernel; a token's
+    matrix ``w [experts, k]``: the product in float32 (plus ``bias``, one number an expert),
+    softmax over all experts, the ``top`` largest scores over their sum (+ 1e-20) times ``scale``
+    (which is the softmax over the chosen logits alone), 0 elsewhere.  One kernel; a token's
     result does not depend on the rest of the step."""
     tokens, k = x.shape
     experts = w.shape[0]
@@ -308,8 +309,11 @@ def router(x: torch.Tensor, w: torch.Tensor, top: int, scale: float) -> torch.Te
     _need(w, "router matrix", torch.float32, (experts, k))
     if not 1 <= top <= experts <= ROUTE_MAX_EXPERTS:
         raise KernelError(f"the router kernel chooses 1 to {experts} of at most {ROUTE_MAX_EXPERTS} experts, not {top}")
+    if bias is not None:
+        _need(bias, "router bias", torch.float32, (experts,))
     out = torch.empty((tokens, experts), dtype=torch.float32, device=x.device)
-    _ok(core().rl_router(_p(x), _p(w), _p(out), tokens, k, experts, top, ctypes.c_float(scale), _tag(x.dtype), _stream()),
+    _ok(core().rl_router(_p(x), _p(w), _p(out), tokens, k, experts, top, ctypes.c_float(scale), _p(bias),
+                         _tag(x.dtype), _stream()),
         "rl_router")
     return out
 
@@ -317,10 +321,13 @@ def router(x: torch.Tensor, w: torch.Tensor, top: int, scale: float) -> torch.Te
 GLU_ALPHA = 1.702  # the sigmoid's slope in the clamped gated activation
 
 
-def swiglu(gate_up: torch.Tensor, out: torch.Tensor, limit: float = 0.0, alpha: float = GLU_ALPHA) -> None:
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor, limit: float = 0.0, alpha: float = GLU_ALPHA,
+           route: Optional[torch.Tensor] = None, expert_ff: int = 0) -> None:
     """The gated activation of a packed ``[gate | up]`` row.  ``limit`` 0: ``silu(g) * u``.
     ``limit > 0``: ``g' * sigmoid(alpha g') * (u' + 1)`` with ``g' = min(g, limit)`` and
-    ``u' = clamp(u, -limit, limit)``."""
+    ``u' = clamp(u, -limit, limit)``.  With ``route`` (float32 ``[tokens, experts]``) the first
+    ``experts * expert_ff`` hidden units are those of the experts side by side and expert ``e``'s
+    are multiplied by ``route[t, e]``."""
     tokens, two_i = gate_up.shape
     if limit < 0:
         raise KernelError(f"the gated activation's limit must not be negative, got {limit}")
@@ -328,10 +335,16 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor, limit: float = 0.0, alpha: 
         raise KernelError(f"the packed [gate | up] row must have even width, has {two_i}")
     _need(gate_up, "gate_up")
     _need(out, "out", gate_up.dtype, (tokens, two_i // 2))
+    experts = 0
+    if route is not None:
+        experts = route.shape[1]
+        _need(route, "route", torch.float32, (tokens, experts))
+        if expert_ff < 1 or experts * expert_ff > two_i // 2:
+            raise KernelError(f"{experts} experts of {expert_ff} hidden units do not fit rows of {two_i // 2}")
     _ok(
         core().rl_swiglu(
             _p(gate_up), _p(out), tokens, two_i // 2, _tag(out.dtype), ctypes.c_float(limit),
-            ctypes.c_float(alpha), _stream(),
+            ctypes.c_float(alpha), _p(route), experts, int(expert_ff), _stream(),
         ),
         "rl_swiglu",
     )
@@ -502,10 +515,13 @@ def attention_generic(
     value_dim: Optional[int] = None,
     keep_first: int = 0,
     sink: bool = False,
+    sink_values: Optional[torch.Tensor] = None,
 ) -> None:
     tokens = q.shape[0]
     pages = k_cache.shape[0]
     dv = d if value_dim is None else int(value_dim)
+    if sink_values is not None:
+        _need(sink_values, "sink values", torch.float32, (nq,))
     _need(q, "q", None, (tokens, nq * d))
     _need(out, "out", q.dtype, (tokens, nq * dv))
     _need(k_cache, "k_cache", q.dtype, (pages, nkv, page_size, d))
@@ -522,9 +538,194 @@ def attention_generic(
         core().rl_attention_generic(
             _p(q), _p(k_cache), _p(v_cache), _p(out), _p(positions), _p(token_slot),
             _p(block_table), block_table.stride(0), page_size, tokens, nq, nkv, d, window,
-            ctypes.c_float(scale), dv, int(keep_first), int(bool(sink)), _tag(q.dtype), _stream(),
+            ctypes.c_float(scale), dv, int(keep_first), int(bool(sink) or sink_values is not None),
+            _p(sink_values), _tag(q.dtype), _stream(),
         ),
         "rl_attention_generic",
+    )
+
+
+def add_layernorm(
+    residual: torch.Tensor,
+    delta1: Optional[torch.Tensor],
+    delta2: Optional[torch.Tensor],
+    weight1: Optional[torch.Tensor],
+    bias1: Optional[torch.Tensor],
+    out1: Optional[torch.Tensor],
+    weight2: Optional[torch.Tensor] = None,
+    bias2: Optional[torch.Tensor] = None,
+    out2: Optional[torch.Tensor] = None,
+    eps: float = 1e-5,
+    rows: Optional[torch.Tensor] = None,
+) -> None:
+    """``residual += delta1 + delta2`` (float32, in place; either may be ``None``), then
+    ``out1 = layernorm(residual) * weight1 + bias1`` and, with ``out2``, a second layer norm of
+    the same rows under ``weight2`` and ``bias2``: the statistics (mean, and the mean of the
+    squared deviations from it) are computed once.  ``out1`` ``None``: only the add.  ``rows`` as
+    in :func:`add_rmsnorm`."""
+    tokens, hidden = residual.shape
+    _need(residual, "residual", torch.float32)
+    out_rows = tokens if rows is None else rows.numel()
+    dtype = None
+    for out, w, b, name in ((out1, weight1, bias1, "first"), (out2, weight2, bias2, "second")):
+        if out is None:
+            continue
+        _need(out, f"{name} output", dtype, (out_rows, hidden))
+        dtype = out.dtype
+        _need(w, f"{name} norm weight", torch.float32, (hidden,))
+        _need(b, f"{name} norm bias", torch.float32, (hidden,))
+    if out2 is not None and out1 is None:
+        raise KernelError("a second layer norm comes with a first")
+    for d in (delta1, delta2):
+        if d is not None:
+            _need(d, "delta", dtype, (tokens, hidden))
+            dtype = d.dtype
+    if dtype is None:
+        return  # nothing to add and nothing to produce
+    if rows is not None:
+        _need(rows, "rows", torch.int32)
+    _ok(
+        core().rl_add_layernorm(
+            _p(residual), _p(delta1), _p(delta2), _p(weight1), _p(bias1), _p(out1), _p(weight2), _p(bias2),
+            _p(out2), _p(rows), out_rows, hidden, ctypes.c_float(eps), _tag(dtype), _stream(),
+        ),
+        "rl_add_layernorm",
+    )
+
+
+def latent_rows(
+    packed: torch.Tensor,
+    q_rank: int,
+    q_norm_w: Optional[torch.Tensor],
+    q_latent_out: Optional[torch.Tensor],
+    kv_col: int,
+    kv_rank: int,
+    rot_dim: int,
+    kv_norm_w: Optional[torch.Tensor],
+    cos: Optional[torch.Tensor],
+    sin: Optional[torch.Tensor],
+    k_cache: Optional[torch.Tensor],
+    v_cache: Optional[torch.Tensor],
+    positions: torch.Tensor,
+    token_slot: torch.Tensor,
+    block_table: torch.Tensor,
+    page_size: int,
+    eps: float,
+    max_position: int,
+) -> None:
+    """From the packed rows of a latent mixer's first product: with ``q_rank`` the query latent
+    (columns ``[0, q_rank)``) RMS-normed under ``q_norm_w`` into ``q_latent_out``; with caches the
+    key/value latent (``kv_rank`` columns from ``kv_col``) RMS-normed under ``kv_norm_w`` and the
+    ``rot_dim`` columns behind it, whose first ``2 * cos.shape[1]`` channels rotate as interleaved
+    pairs, written to the token's place: ``k_cache [pages, 1, page, kv_rank + rot_dim]`` holds
+    ``[latent | rotated part]``, ``v_cache [pages, 1, kv_rank, page]`` the latent transposed."""
+    tokens, row_width = packed.shape
+    _need(packed, "packed rows")
+    _need(positions, "positions", torch.int32, (tokens,))
+    _need(token_slot, "token_slot", torch.int32, (tokens,))
+    _need(block_table, "block_table", torch.int32)
+    if q_rank:
+        _need(q_norm_w, "query latent norm weight", torch.float32, (q_rank,))
+        _need(q_latent_out, "query latent", packed.dtype, (tokens, q_rank))
+        if q_rank > row_width:
+            raise KernelError(f"a query latent of {q_rank} columns in rows of {row_width}")
+    half = 0
+    if k_cache is not None:
+        pages = k_cache.shape[0]
+        _need(k_cache, "k_cache", packed.dtype, (pages, 1, page_size, kv_rank + rot_dim))
+        _need(v_cache, "v_cache", packed.dtype, (pages, 1, kv_rank, page_size))
+        _need(kv_norm_w, "latent norm weight", torch.float32, (kv_rank,))
+        if kv_col < 0 or kv_col + kv_rank + rot_dim > row_width or rot_dim % 2:
+            raise KernelError(
+                f"a latent of {kv_rank} + {rot_dim} columns from column {kv_col} in rows of {row_width}"
+            )
+        if max_position // page_size >= block_table.shape[1]:
+            raise KernelError(
+                f"position {max_position} needs page {max_position // page_size} of a block table "
+                f"with {block_table.shape[1]} columns"
+            )
+        if cos is not None:
+            half = cos.shape[1]
+            _need(cos, "cos table", torch.float32, (None, half))
+            _need(sin, "sin table", torch.float32, tuple(cos.shape))
+            if 2 * half > rot_dim or max_position >= cos.shape[0]:
+                raise KernelError(
+                    f"rotation tables of {half} pairs and {cos.shape[0]} positions for a part of {rot_dim} "
+                    f"channels at position {max_position}"
+                )
+    _ok(
+        core().rl_latent_rows(
+            _p(packed), row_width, tokens, int(q_rank), _p(q_norm_w), _p(q_latent_out), int(kv_col), int(kv_rank),
+            int(rot_dim), _p(kv_norm_w), _p(cos), _p(sin), half, _p(k_cache), _p(v_cache), _p(positions),
+            _p(token_slot), _p(block_table), block_table.stride(0), page_size, ctypes.c_float(eps),
+            _tag(packed.dtype), _stream(),
+        ),
+        "rl_latent_rows",
+    )
+
+
+def rotate_tail(
+    q: torch.Tensor, out: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
+    positions: torch.Tensor, heads: int, d: int, rot_dim: int, out_width: int, offset: int, max_position: int,
+) -> None:
+    """``out[t, h, offset : offset + rot_dim]`` = the last ``rot_dim`` channels of head ``h`` of
+    ``q`` (rows that begin with ``heads * (d + rot_dim)`` channels and may be wider), the first
+    ``2 * cos.shape[1]`` of them rotated as interleaved pairs by the token's position; ``out`` has
+    ``out_width`` channels a head."""
+    tokens = q.shape[0]
+    _need(q, "q", None, (tokens, None))
+    if q.shape[1] < heads * (d + rot_dim):
+        raise KernelError(f"rows of {q.shape[1]} channels do not hold {heads} heads of {d} + {rot_dim}")
+    _need(out, "out", q.dtype, (tokens, heads * out_width))
+    _need(positions, "positions", torch.int32, (tokens,))
+    half = 0
+    if cos is not None:
+        half = cos.shape[1]
+        _need(cos, "cos table", torch.float32, (None, half))
+        _need(sin, "sin table", torch.float32, tuple(cos.shape))
+        if max_position >= cos.shape[0]:
+            raise KernelError(f"position {max_position} is beyond the rotation table of {cos.shape[0]} positions")
+    if rot_dim % 2 or 2 * half > rot_dim or offset < 0 or offset + rot_dim > out_width:
+        raise KernelError(f"{rot_dim} channels ({half} pairs rotate) at {offset} of heads of {out_width}")
+    _ok(
+        core().rl_rotate_tail(
+            _p(q), _p(out), _p(cos), _p(sin), _p(positions), tokens, heads, d, rot_dim, half, out_width, offset,
+            q.shape[1], _tag(q.dtype), _stream(),
+        ),
+        "rl_rotate_tail",
+    )
+
+
+def head_product(
+    x: torch.Tensor, w: torch.Tensor, y: torch.Tensor, heads: int, x_head: int, x_off: int, y_head: int, y_off: int,
+    gate: Optional[torch.Tensor] = None, gate_col: int = 0,
+) -> None:
+    """``y[t, y_off + h * y_head + o] = sum_i w[h, o, i] * x[t, x_off + h * x_head + i]``: one small
+    matrix a head (``w [heads, O, I]``), applied to a slice of every head of ``x`` and written into
+    a slice of every head of ``y``.  ``gate``: the result is multiplied by
+    ``sigmoid(gate[t, gate_col + h])``.  Sizes in steps of 16 (and offsets in steps of 4) run on
+    the matrix cores, in the type of the operands (float32: the true 32-bit instruction)."""
+    tokens = x.shape[0]
+    _need(x, "x", None, (tokens, None))
+    _need(y, "y", x.dtype, (tokens, None))
+    _need(w, "head matrices", x.dtype, (heads, None, None))
+    O, I = w.shape[1], w.shape[2]
+    if x_off < 0 or x_off + (heads - 1) * x_head + I > x.shape[1]:
+        raise KernelError(f"{heads} heads of {I} inputs every {x_head} from {x_off} lie outside rows of {x.shape[1]}")
+    if y_off < 0 or y_off + (heads - 1) * y_head + O > y.shape[1]:
+        raise KernelError(f"{heads} heads of {O} outputs every {y_head} from {y_off} lie outside rows of {y.shape[1]}")
+    gate_row = 0
+    if gate is not None:
+        _need(gate, "gate", x.dtype, (tokens, None))
+        gate_row = gate.shape[1]
+        if not 0 <= gate_col <= gate_row - heads:
+            raise KernelError(f"gate columns {gate_col}..{gate_col + heads} lie outside rows of {gate_row}")
+    _ok(
+        core().rl_head_product(
+            _p(x), _p(w), _p(y), tokens, heads, I, O, x.shape[1], x_head, x_off, y.shape[1], y_head, y_off,
+            _p(gate), gate_row, gate_col, _tag(x.dtype), _stream(),
+        ),
+        "rl_head_product",
     )
 
 
@@ -1242,12 +1443,17 @@ def attention_tile(
     keep_first: int,
     sink: bool,
     scale: float,
+    sink_values: Optional[torch.Tensor] = None,
 ) -> None:
     """Attention of every token of the step, in tiles of 16 rows on the matrix cores, for value
     heads of a size of their own, a window that keeps a request's first ``keep_first`` positions
-    visible, and (``sink``) a softmax with 1 added to its denominator.  float32 (bit for bit the
+    visible, and (``sink``) a softmax with 1 added to its denominator, or with ``sink_values``
+    (float32, one number a query head) ``exp`` of the head's number.  float32 (bit for bit the
     same however the step was cut) or bfloat16."""
     tokens = q.shape[0]
+    if sink_values is not None:
+        _need(sink_values, "sink values", torch.float32, (nq,))
+        sink = True
     pages = k_cache.shape[0]
     _need(q, "q", None, (tokens, nq * d))
     _need(out, "out", q.dtype, (tokens, nq * dv))
@@ -1285,7 +1491,7 @@ def attention_tile(
             _p(q), _p(k_cache), _p(v_cache), _p(out), _p(tiles), num_tiles, _p(ctx.positions),
             _p(ctx.token_slot), _p(block_table), block_table.stride(0), page_size, nq, nkv, window,
             int(keep_first), int(bool(sink)), ctypes.c_float(scale), nsplit, _p(part), tokens, tile_rows,
-            _tag(q.dtype), _stream(),
+            _tag(q.dtype), _p(sink_values), _stream(),
         ),
         "rl_attn_tile",
     )
@@ -1321,6 +1527,7 @@ def paged_attention(
     value_dim: Optional[int] = None,
     keep_first: int = 0,
     sink: bool = False,
+    sink_values: Optional[torch.Tensor] = None,
 ) -> None:
     """Attention of every token of the step over its request's cached keys.
 
@@ -1334,23 +1541,24 @@ def paged_attention(
 
     ``value_dim`` (the size of a value head, where it is not ``d``), ``keep_first`` (with a window:
     the request's first positions stay visible behind it) and ``sink`` (1 added to the softmax's
-    denominator: a key of score 0 without a value) send the step to the kernels that take them:
+    denominator: a key of score 0 without a value; with ``sink_values`` its score is a number of
+    the query head, not scaled) send the step to the kernels that take them:
     tiles of 16 rows on the matrix cores for head sizes in steps of 16, the FMA kernel otherwise."""
     if prepare is not None and not attention_prepares_queries(q.dtype, d, 0 if prepare[1] is None else prepare[1].shape[1]):
         raise KernelError("the attention kernels do not finish the queries of this head size, type or rotation")
     dv = d if value_dim is None else int(value_dim)
     keep_first = int(keep_first) if window > 0 else 0  # without a window every key is seen anyway
-    if dv != d or keep_first or sink:
+    if dv != d or keep_first or sink or sink_values is not None:
         # value heads of their own size, kept first positions, one more term in the denominator
         if prepare is not None:
             raise KernelError("queries are finished before an attention with these options")
         if d % 16 == 0 and dv % 16 == 0 and page_size % 4 == 0:
             attention_tile(q, k_cache, v_cache, out, ctx, block_table, page_size, nq, nkv, d, dv,
-                           window, keep_first, sink, scale)
+                           window, keep_first, sink, scale, sink_values)
         else:
             attention_generic(
                 q, k_cache, v_cache, out, ctx.positions, ctx.token_slot, block_table, page_size,
-                nq, nkv, d, window, scale, ctx.max_position, dv, keep_first, sink,
+                nq, nkv, d, window, scale, ctx.max_position, dv, keep_first, sink, sink_values,
             )
         return
     if q.dtype == torch.float32 and d % 16 == 0:

@@ -10,7 +10,7 @@ next norm kernel, as the reference threads ``(hidden, residual)`` through its la
 from __future__ import annotations
 
 from .base import BLOCKS, Block
-from .lazy import NormedDelta, plain, run_norm
+from .lazy import NormedDelta, SummedDeltas, plain, run_norm
 
 
 class PreNormBlock(Block):
@@ -76,5 +76,41 @@ class SandwichBlock(Block):
         return self._pending(self.feed_forward_post_norm, self.feed_forward.forward(x, ctx))
 
 
+class ParallelBlock(Block):
+    """Both sub-layers read the same stream: ``r += mixer(norm1(r)) + feed_forward(norm2(r))``.
+    Their outputs travel on as one pending :class:`~rapid_llm_amd.parts.lazy.SummedDeltas`; where
+    the two norms can share their statistics (``pairs_with``) one kernel adds what is pending
+    and writes both sub-layers' inputs."""
+
+    replayable = True
+    accepts_deferred = True
+
+    def __init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm) -> None:
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.mixer_norm = mixer_norm
+        self.feed_forward_norm = feed_forward_norm
+
+    def parts(self):
+        if self.feed_forward is None:
+            return (self.mixer_norm, self.mixer)
+        return (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward)
+
+    def forward(self, residual, delta, ctx, cache):
+        if self.feed_forward is None:
+            x = run_norm(self.mixer_norm, residual, delta, ctx)
+            return self.mixer.forward(x, ctx, cache)
+        pairs = getattr(self.mixer_norm, "pairs_with", None)
+        if pairs is not None and pairs(self.feed_forward_norm):
+            x1, x2 = self.mixer_norm.forward(residual, delta, ctx, second=self.feed_forward_norm)
+        else:
+            x1 = plain(run_norm(self.mixer_norm, residual, delta, ctx))
+            x2 = plain(run_norm(self.feed_forward_norm, residual, None, ctx))
+        a = self.mixer.forward(x1, ctx, cache)
+        b = self.feed_forward.forward(x2, ctx)
+        return SummedDeltas(a, b)
+
+
+BLOCKS.register("parallel", ParallelBlock)
 BLOCKS.register("prenorm", PreNormBlock)
 BLOCKS.register("sandwich", SandwichBlock)

@@ -19,6 +19,11 @@ products on either side absorb it, without any part knowing its neighbours:
   to the stream and computes its own rows in one kernel; anything else gets the normed rows in
   the stream's type from ``materialize()``.
 
+* :class:`SummedDeltas`: what a block whose two sub-layers read the same stream returns: both
+  outputs, not yet added to each other.  A norm that declares ``fuses_products`` and knows the
+  type adds both into the stream in the kernel that computes its own rows; anything else gets
+  their sum joined to the stream first (``add_to``) or as a tensor (``materialize``).
+
 Blocks and models route these only between parts that declare them (``fuses_products`` on
 a norm, ``accepts_scaled_rows`` on a mixer or feed-forward, ``accepts_deferred`` on a
 block); everything else sees plain tensors.
@@ -70,6 +75,35 @@ class NormedDelta:
         return out
 
 
+class SummedDeltas:
+    """``first + second``, the outputs of two sub-layers that read the same stream, not yet added."""
+
+    def __init__(self, first, second) -> None:
+        self.first = first
+        self.second = second
+
+    @property
+    def shape(self):
+        return self.first.shape
+
+    def tensors(self) -> tuple[torch.Tensor, torch.Tensor]:
+        return plain(self.first), plain(self.second)
+
+    def add_to(self, residual: torch.Tensor) -> None:
+        """``residual += first + second`` in place (float32)."""
+        from ..kernels import ops
+
+        a, b = self.tensors()
+        ops.add_layernorm(residual, a, b, None, None, None)
+
+    def materialize(self, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+        """The sum as a float32 tensor."""
+        a, _ = self.tensors()
+        out = torch.zeros(a.shape, dtype=torch.float32, device=a.device)
+        self.add_to(out)
+        return out
+
+
 @dataclass
 class ScaledRows:
     rows: torch.Tensor  # [M, size], the residual rows times the norm's weight
@@ -92,13 +126,13 @@ class ScaledRows:
 
 def plain(value):
     """A tensor, whatever lazy value it still was."""
-    return value.materialize() if isinstance(value, (DeferredProduct, NormedDelta)) else value
+    return value.materialize() if isinstance(value, (DeferredProduct, NormedDelta, SummedDeltas)) else value
 
 
 def settle(residual, delta):
     """What is left to add once lazy values are settled: a pending normed delta joins the stream
     now, a deferred product becomes a tensor."""
-    if isinstance(delta, NormedDelta):
+    if isinstance(delta, (NormedDelta, SummedDeltas)):
         delta.add_to(residual)
         return None
     return plain(delta)
@@ -110,7 +144,7 @@ def run_norm(norm, residual, delta, ctx, consumer=None, rows=None):
         return norm.forward(
             residual, delta, ctx, rows, scaled_ok=bool(getattr(consumer, "accepts_scaled_rows", False))
         )
-    if isinstance(delta, NormedDelta):
+    if isinstance(delta, (NormedDelta, SummedDeltas)):
         # a norm that knows nothing of it: the stream takes it first
         delta.add_to(residual)
         delta = None

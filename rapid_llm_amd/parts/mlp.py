@@ -121,8 +121,11 @@ class TwoLayer(FeedForward):
 
 class RoutedExperts(FeedForward):
     """A mixture of two-layer experts: every token uses the ``top`` experts that a softmax router
-    scores highest, weighted by their scores over the chosen ones' sum, times ``route_scale``;
-    a shared expert (``shared_size`` > 0) runs for every token and is added.
+    scores highest, weighted by their scores over the chosen ones' sum (which is the softmax over
+    the chosen logits alone), times ``route_scale``; a shared expert (``shared_size`` > 0) runs for
+    every token and is added.  ``gated``: the experts are gated ones, ``down(silu(gate(x)) * up(x))``;
+    their gate and up projections form one packed matrix, all gates first.  ``router_bias_name``:
+    the router's logits get a bias, one number an expert.
 
     The router's product and scores are float32 in every engine (its matrix is held in
     float32).  The experts' up projections are one packed matrix ``[experts * expert_size +
@@ -151,9 +154,18 @@ class RoutedExperts(FeedForward):
         shared_prefix: str = "shared.",
         up_name: str = "up",
         down_name: str = "down",
+        gated: bool = False,
+        gate_name: str = "gate",
+        router_bias_name: str | None = None,
     ) -> None:
-        if activation not in ops.UNARY_ACTIVATIONS:
+        self.gated = bool(gated)
+        if self.gated:
+            if activation != "silu":
+                raise ValueError(f"gated experts use the silu gate, not {activation!r}")
+        elif activation not in ops.UNARY_ACTIVATIONS:
             raise ValueError(f"activation {activation!r} is not one of {sorted(ops.UNARY_ACTIVATIONS)}")
+        self.gate_name, self.router_bias_name = gate_name, router_bias_name
+        self.router_bias = None
         if not 1 <= top <= num_experts <= ops.ROUTE_MAX_EXPERTS:
             raise ValueError(f"a token uses 1 to {num_experts} of at most {ops.ROUTE_MAX_EXPERTS} experts, not {top}")
         self.hidden_size, self.num_experts, self.top = hidden_size, num_experts, top
@@ -163,7 +175,7 @@ class RoutedExperts(FeedForward):
         self.names = (router_name, expert_prefix, shared_prefix, up_name, down_name)
         self.inner = num_experts * expert_size + shared_size
         self.router = Linear(hidden_size, num_experts)
-        self.up = Linear(hidden_size, self.inner)
+        self.up = Linear(hidden_size, (2 if self.gated else 1) * self.inner)
         self.down = Linear(self.inner, hidden_size)
 
     def _sources(self, which: str, rows_of_expert: int, rows_of_shared: int) -> tuple[Source, ...]:
@@ -176,22 +188,36 @@ class RoutedExperts(FeedForward):
     def param_specs(self) -> list[ParamSpec]:
         h = self.hidden_size
         router, _, _, up, down = self.names
-        return [
+        first = self._sources(up, self.expert_size, self.shared_size)
+        if self.gated:  # [every gate | every up]
+            first = self._sources(self.gate_name, self.expert_size, self.shared_size) + first
+        specs = [
             ParamSpec(self.name + ".router", (self.num_experts, h), "matrix_f32",
                       (Source(self.prefix + router, self.num_experts),)),
-            ParamSpec(self.name + ".up", (self.inner, h), "matrix", self._sources(up, self.expert_size, self.shared_size)),
+            ParamSpec(self.name + ".up", (self.up.out_features, h), "matrix", first),
             ParamSpec(self.name + ".down", (h, self.inner), "matrix",
                       self._sources(down, self.expert_size, self.shared_size), axis=1),
         ]
+        if self.router_bias_name:
+            specs.append(ParamSpec(self.name + ".router_bias", (self.num_experts,), "vector",
+                                   (Source(self.prefix + self.router_bias_name, self.num_experts),)))
+        return specs
 
     def bind(self, params, runtime) -> None:
+        if self.router_bias_name:
+            self.router_bias = params[self.name + ".router_bias"]
         self.router.bind(params[self.name + ".router"])
         self.up.bind(params[self.name + ".up"])
         self.down.bind(params[self.name + ".down"])
 
     def forward(self, x, ctx):
-        weights = ops.router(x, self.router.weight, self.top, self.route_scale)  # float32 throughout
+        # float32 throughout
+        weights = ops.router(x, self.router.weight, self.top, self.route_scale, self.router_bias)
         hidden = self.up(x)
+        if self.gated:
+            act = torch.empty((x.shape[0], self.inner), dtype=hidden.dtype, device=x.device)
+            ops.swiglu(hidden, act, route=weights, expert_ff=self.expert_size)
+            return self.down.deferred(act, ctx)
         ops.unary_act(hidden, hidden, self.activation, weights, self.expert_size)
         return self.down.deferred(hidden, ctx)
 
