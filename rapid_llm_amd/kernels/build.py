@@ -55,7 +55,10 @@ HEADERS = ("common.h", "static_entry.h")
 DEFAULT_HEAD_DIMS = tuple(range(16, 257, 16))
 
 # pairs of (key, value) head sizes of the tile attention that build_all() builds ahead of time
-DEFAULT_TILE_HEAD_DIMS = ((16, 16), (16, 48), (32, 16), (32, 32), (64, 32), (64, 64), (64, 128), (128, 64), (128, 128))
+DEFAULT_TILE_HEAD_DIMS = (
+    (16, 16), (16, 48), (32, 16), (32, 32), (48, 32), (64, 32), (64, 64), (64, 128), (96, 80), (128, 64), (128, 96),
+    (128, 128), (160, 144), (320, 256),
+)
 
 _HIPCC_FLAGS = (
     "-O3",
@@ -224,9 +227,11 @@ def mlstm_library(force: bool = False) -> Path:
 
 
 def attention_tile_library(head_dim: int, value_dim: int, force: bool = False) -> Path:
-    for size in (head_dim, value_dim):
-        if size % 16 or not 16 <= size <= 256:
-            raise KernelBuildError(f"the tile attention takes head sizes in steps of 16 up to 256, got {size}")
+    # beyond 320 / 256 channels a lane's operands no longer fit its registers: the compiler
+    # parks some in scratch memory, which is slower and as exact
+    for size, most in ((head_dim, 576), (value_dim, 512)):
+        if size % 16 or not 16 <= size <= most:
+            raise KernelBuildError(f"the tile attention takes head sizes in steps of 16 up to {most}, got {size}")
     flags = (f"-DRL_HEAD_DIM={head_dim}", f"-DRL_VALUE_DIM={value_dim}", "-mllvm", "-amdgpu-mfma-vgpr-form=1")
     return compile_library(f"attn_tile_d{head_dim}_v{value_dim}", ATTENTION_TILE_SOURCES, flags, force=force)
 
@@ -234,7 +239,8 @@ def attention_tile_library(head_dim: int, value_dim: int, force: bool = False) -
 def build_all(head_dims: tuple[int, ...] = DEFAULT_HEAD_DIMS, force: bool = True) -> list[Path]:
     """Compile every library (what ``__graft_entry__.build`` calls)."""
     out = [core_library(force=force), mlstm_library(force=force)]
-    out += [attention_tile_library(d, dv, force=force) for d, dv in DEFAULT_TILE_HEAD_DIMS]
+    with ThreadPoolExecutor(8) as pool:
+        out += list(pool.map(lambda pair: attention_tile_library(*pair, force=force), DEFAULT_TILE_HEAD_DIMS))
     if not all((CSRC / s).is_file() for s in ATTENTION_SOURCES):
         return out
     with ThreadPoolExecutor(min(8, len(head_dims))) as pool:

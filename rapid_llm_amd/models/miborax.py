@@ -12,7 +12,7 @@ from __future__ import annotations
 
 from ..config.miborax import MiboraxConfig
 from ..config.registry import register_architecture
-from .spec import LayerSpec, ModelSpec, PartSpec, linear_output, token_embedding_scaled
+from .spec import IgnoreRule, LayerSpec, ModelSpec, PartSpec, linear_output, token_embedding_scaled
 
 
 def build_miborax_spec(cfg: MiboraxConfig) -> ModelSpec:
@@ -21,6 +21,7 @@ def build_miborax_spec(cfg: MiboraxConfig) -> ModelSpec:
                                       "bias_checkpoint_name": name + ".b"})
 
     layers = []
+    unread = []
     for i, layer in enumerate(cfg.layers):
         prefix = f"l{i}."
         m = layer.mixer
@@ -49,6 +50,10 @@ def build_miborax_spec(cfg: MiboraxConfig) -> ModelSpec:
                 },
             )
             ff_norm = norm(prefix + "norm2")
+        else:
+            # a checkpoint may still carry the second norm of a layer without a feed-forward:
+            # nothing reads its output
+            unread.append(IgnoreRule(rf"l{i}\.norm2(\.b)?"))
         layers.append(
             LayerSpec(
                 mixer=mixer, feed_forward=ff, mixer_norm=norm(prefix + "norm1"), feed_forward_norm=ff_norm,
@@ -64,6 +69,7 @@ def build_miborax_spec(cfg: MiboraxConfig) -> ModelSpec:
         embedding=token_embedding_scaled(cfg.vocab, cfg.width, "embed", cfg.embedding_scale),
         # the output projection is the embedding's table: the checkpoint ships no tensor of its own
         output=linear_output(cfg.vocab, cfg.width, "head", tied=True),
+        ignore_tensors=tuple(unread),
     )
 
 
