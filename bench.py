@@ -3,7 +3,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--dtype bfloat16]
                     [--shape NAME] [--batch B] [--prompt-len T] [--context C]
     python bench.py --workload qwen3-0.6b-256 | qwen3-32b-32
-    python bench.py --design fokulorn|sikevik [--design-size 2b,8b]
+    python bench.py --design fokulorn|sikevik|miborax [--design-size 2b,8b]
 
 A "step" is one decode step of the whole batch through the engine's step function and the
 greedy sampling kernel, tokens fed back.  The default run has the layer sizes of
@@ -35,6 +35,12 @@ request's first positions, with a sink term and value heads of half the key head
 before and behind every sub-layer; one dense two-layer feed-forward, then mixtures of eight
 experts with a shared one; the last six layers in two passes of three), whose feed-forward
 matrices hold as many weights a layer as Qwen3's.
+
+``--design miborax`` does the same for the Miborax decoder (attention through a latent row that
+all heads share, half of the layers windowed, a quarter reading the rows another layer cached; both
+sub-layers of a layer behind layer norms of the same stream; mixtures of eight gated experts with a
+router bias), beside the Sikevik decoder, the engine's closest (a sink term, windows, routed
+experts), and Qwen3 of equal size.
 
 Metric definitions follow rapid_llm's docs/benchmark_models.md:141-149: decode tok/s is
 batch / mean step time; prefill tok/s is prompt tokens / prefill latency; both timed
@@ -506,9 +512,152 @@ def _time_kernels(z: dict, prompt_len: int, batch: int) -> dict:
     }
 
 
+# Latent sizes for ``--design miborax``: a row of 256 channels and a rotated part of 64 that all
+# heads share, heads of 128 + 64 query channels and 128 value channels, queries through a latent of
+# three quarters of the width in the layers that see everything.
+MIBORAX_LATENT = dict(kv_rank=256, rot_dim=64, dim=128, vdim=128)
+
+
+def miborax_body(z: dict) -> dict:
+    """Of every four layers the first and last are windowed with rows of their own, the second sees
+    everything and takes its queries through a latent, the third is windowed and reads the first's
+    rows.  Eight gated experts of an eighth of Qwen3's feed-forward width each (two of eight used):
+    a layer's feed-forward matrices hold what Qwen3's three do."""
+    lat = MIBORAX_LATENT
+    scale = (lat["dim"] + lat["rot_dim"]) ** -0.5
+
+    def mixer(**more):
+        return {"heads": z["heads"], "dim": lat["dim"], "rot_dim": lat["rot_dim"], "vdim": lat["vdim"],
+                "kv_rank": lat["kv_rank"], "scale": scale, "rot": {"base": 10000.0, "dims": lat["rot_dim"]}, **more}
+
+    moe = {"kind": "moe", "expert": {"ff": z["ff"] // 8}, "router": {"experts": 8, "top": 2}}
+    layers = []
+    for i in range(z["layers"]):
+        if i % 4 == 1:
+            layers.append({"type": "latent_attention", "mixer": mixer(q_rank=z["width"] * 3 // 4), "mlp": moe})
+        elif i % 4 == 2:
+            layers.append({"type": "latent_attention_2", "mixer": mixer(mask={"size": z["window"]}, kv_from=i - 2), "mlp": moe})
+        else:
+            layers.append({"type": "latent_attention_2", "mixer": mixer(mask={"size": z["window"]}), "mlp": moe})
+    return {"architecture": "Miborax", "width": z["width"], "vocab": z["vocab"], "embedding": {"scale": 1.0},
+            "norm": {"eps": 1e-6}, "layers": layers}
+
+
+def _time_calls(call, graph: bool) -> float:
+    """Seconds a call.  ``graph``: ten calls recorded and replayed, as a decode step runs them
+    (launched one by one, short kernels cost the host more than the device)."""
+    import torch
+
+    for _ in range(3):
+        call()
+    torch.cuda.synchronize()
+    if graph:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(10):
+                call()
+        g.replay()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(5):
+            g.replay()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) / 50
+    t = time.perf_counter()
+    for _ in range(10):
+        call()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t) / 10
+
+
+def _time_miborax_kernels(z: dict, prompt_len: int, batch: int) -> dict:
+    """The design's own kernels alone, microseconds and share of the roofline each.  Attention over
+    the shared rows: one prompt from its start (matrix rate over the keys every query sees, each a
+    row of ``kv_rank + rot_dim`` channels against ``heads`` queries, and ``kv_rank`` channels of
+    values) and ``batch`` single tokens behind ``prompt_len`` (bytes of the rows read: the latent
+    twice, once as keys and once transposed as values), windowed and over everything.  The heads'
+    key and value matrices (matrix rate in a prompt step, bytes of the matrices in a decode step)
+    and the pair of layer norms with the residual add (bytes)."""
+    import types
+
+    import torch
+
+    from rapid_llm_amd.kernels import ops
+
+    lat = MIBORAX_LATENT
+    nq, r, rd, dn, dv, page, dev = z["heads"], lat["kv_rank"], lat["rot_dim"], lat["dim"], lat["vdim"], 16, "cuda"
+    d = r + rd
+    sink = torch.zeros(nq, device=dev)
+    out = {}
+
+    def attention(seqs, window):
+        tokens = sum(n for _, n in seqs)
+        per = -(-max(a + n for a, n in seqs) // page)
+        pages = len(seqs) * per + 1
+        table = (1 + torch.arange(len(seqs) * per, dtype=torch.int32, device=dev)).view(len(seqs), per).contiguous()
+        kc = (torch.randn(pages, 1, page, d, device=dev) * 0.5).bfloat16()
+        vc = (torch.randn(pages, 1, r, page, device=dev) * 0.5).bfloat16()
+        q = (torch.randn(tokens, nq * d, device=dev) * 0.5).bfloat16()
+        res = torch.empty((tokens, nq * r), dtype=torch.bfloat16, device=dev)
+        pos = torch.cat([torch.arange(a, a + n, dtype=torch.int32) for a, n in seqs]).to(dev)
+        slot = torch.cat([torch.full((n,), i, dtype=torch.int32) for i, (_, n) in enumerate(seqs)]).to(dev)
+        ctx = types.SimpleNamespace(positions=pos, token_slot=slot, token_ids=pos, h_seq_starts=[a for a, _ in seqs],
+                                    h_seq_lens=[n for _, n in seqs], max_position=int(pos.max()), extra={})
+        return _time_calls(lambda: ops.paged_attention(q, kc, vc, res, ctx, table, page, nq, 1, d, window, d ** -0.5,
+                                                       value_dim=r, sink_values=sink), graph=False)
+
+    for name, window in (("windowed", z["window"]), ("causal", 0)):
+        sec = attention([(0, prompt_len)], window)
+        seen = sum(min(p + 1, window) if window else p + 1 for p in range(prompt_len))
+        out[f"attention_{name}_prefill_us"] = round(sec * 1e6, 1)
+        out[f"attention_{name}_prefill_frac_bf16_matrix"] = round(
+            2.0 * nq * seen * (d + r) / sec / (PEAK_TFLOPS["bfloat16"] * 1e12), 4)
+        sec = attention([(prompt_len, 1)] * batch, window)
+        keys = min(prompt_len + 1, window) if window else prompt_len + 1
+        out[f"attention_{name}_decode_us"] = round(sec * 1e6, 1)
+        out[f"attention_{name}_decode_frac_hbm"] = round(2.0 * batch * keys * (d + r) / sec / 1e9 / HBM_GBPS, 4)
+
+    # the heads' key matrices (queries into the latent's channels) and value matrices
+    uk = (torch.randn(nq, r, dn, device=dev) * 0.05).bfloat16()
+    uv = (torch.randn(nq, dv, r, device=dev) * 0.05).bfloat16()
+    for what, tokens in (("prefill", prompt_len), ("decode", batch)):
+        q = (torch.randn(tokens, nq * (dn + rd), device=dev) * 0.5).bfloat16()
+        full = torch.empty((tokens, nq * d), dtype=torch.bfloat16, device=dev)
+        mean = (torch.randn(tokens, nq * r, device=dev) * 0.5).bfloat16()
+        heads_out = torch.empty((tokens, nq * dv), dtype=torch.bfloat16, device=dev)
+        small = what == "decode"
+        sec_k = _time_calls(lambda: ops.head_product(q, uk, full, nq, dn + rd, 0, d, 0), graph=small)
+        sec_v = _time_calls(lambda: ops.head_product(mean, uv, heads_out, nq, r, 0, dv, 0), graph=small)
+        flops = 2.0 * tokens * nq * r * dn
+        moved = 2.0 * (nq * r * dn + tokens * nq * (dn + r))
+        for tag, sec, io in (("key", sec_k, moved), ("value", sec_v, 2.0 * (nq * r * dv + tokens * nq * (r + dv)))):
+            out[f"head_{tag}_matrices_{what}_us"] = round(sec * 1e6, 1)
+            if small:
+                out[f"head_{tag}_matrices_{what}_frac_hbm"] = round(io / sec / 1e9 / HBM_GBPS, 4)
+            else:
+                out[f"head_{tag}_matrices_{what}_frac_bf16_matrix"] = round(flops / sec / (PEAK_TFLOPS["bfloat16"] * 1e12), 4)
+
+    # both layer norms of a layer with the add of the two sub-layers' outputs in front
+    width = z["width"]
+    for what, tokens in (("prefill", prompt_len), ("decode", batch)):
+        res = torch.randn(tokens, width, device=dev)
+        d1 = torch.randn(tokens, width, device=dev).bfloat16()
+        d2 = torch.randn(tokens, width, device=dev).bfloat16()
+        w1, b1, w2, b2 = (torch.randn(width, device=dev) for _ in range(4))
+        o1 = torch.empty((tokens, width), dtype=torch.bfloat16, device=dev)
+        o2 = torch.empty_like(o1)
+        sec = _time_calls(lambda: ops.add_layernorm(res, d1, d2, w1, b1, o1, w2, b2, o2, eps=1e-6), graph=what == "decode")
+        out[f"add_two_layernorms_{what}_us"] = round(sec * 1e6, 1)
+        out[f"add_two_layernorms_{what}_frac_hbm"] = round(tokens * width * (4 + 4 + 2 + 2 + 2 + 2) / sec / 1e9 / HBM_GBPS, 4)
+    return out
+
+
+# design -> (name, its configuration at a size, its kernels alone, the engine's closest other
+# architecture measured beside it and Qwen3)
 DESIGNS = {
-    "fokulorn": ("Fokulorn", fokulorn_body, _time_kernels),
-    "sikevik": ("Sikevik", sikevik_body, _time_sikevik_kernels),
+    "fokulorn": ("Fokulorn", fokulorn_body, _time_kernels, None),
+    "sikevik": ("Sikevik", sikevik_body, _time_sikevik_kernels, None),
+    "miborax": ("Miborax", miborax_body, _time_miborax_kernels, ("sikevik", sikevik_body)),
 }
 
 
@@ -516,9 +665,12 @@ def run_design(args) -> int:
     if args.design not in DESIGNS:
         print(f"unknown design {args.design!r}; known: {', '.join(sorted(DESIGNS))}")
         return 2
-    title, design_body, design_kernels = DESIGNS[args.design]
+    title, design_body, design_kernels, closest = DESIGNS[args.design]
     prompt_len = args.prompt_len or 2048
-    out = {"design": title, "beside": "Qwen3 of equal width, depth, heads and feed-forward width",
+    beside = "Qwen3 of equal width, depth, heads and feed-forward width"
+    if closest is not None:
+        beside = f"{closest[0]} and " + beside
+    out = {"design": title, "beside": beside,
            "dtype": "bf16", "data": "synthetic (uniform random token ids, random N(0,0.02) weights)",
            "prompt_len": prompt_len, "batch": args.batch, "sizes": {}}
     for name in [x for x in args.design_size.split(",") if x]:
@@ -526,6 +678,9 @@ def run_design(args) -> int:
         row = {"config": z}
         row[args.design] = _time_model(design_body(z), prompt_len, args.batch, args.point_steps, prompt_len + 512)
         print(f"[bench] {name} {args.design} {row[args.design]}", file=sys.stderr, flush=True)
+        if closest is not None:
+            row[closest[0]] = _time_model(closest[1](z), prompt_len, args.batch, args.point_steps, prompt_len + 512)
+            print(f"[bench] {name} {closest[0]} {row[closest[0]]}", file=sys.stderr, flush=True)
         row["qwen3"] = _time_model(qwen3_body(z), prompt_len, args.batch, args.point_steps, prompt_len + 512)
         print(f"[bench] {name} qwen3 {row['qwen3']}", file=sys.stderr, flush=True)
         row["kernels"] = design_kernels(z, prompt_len, args.batch)
@@ -560,7 +715,7 @@ def main() -> int:
     ap.add_argument("--peaks", action="store_true",
                     help="measure what the device reaches with library kernels (a large read, copy and square products) and exit")
     ap.add_argument("--design", default=None,
-                    help="measure another architecture of the engine beside Qwen3 at equal size (fokulorn, sikevik) and exit")
+                    help="measure another architecture of the engine beside Qwen3 at equal size (fokulorn, sikevik, miborax) and exit")
     ap.add_argument("--design-size", default="2b,8b", help=f"sizes for --design: {', '.join(DESIGN_SIZES)}")
     args = ap.parse_args()
     if args.peaks:

@@ -460,8 +460,10 @@ __global__ __launch_bounds__(AW* RL_WAVE) void attn_tile_kernel(
     }
 }
 
-// Fold the shares of a row's keys that nsplit workgroups left (in order: the same bits every
-// run), add the sink's term and write the row.  One wave a row, a lane a channel (and more).
+// Fold the shares of a row's keys that nsplit (at most 64) workgroups left, in order (the same
+// bits every run), add the sink's term and write the row.  One wave a row: lane s holds share s's
+// maximum and sum, every lane takes them from there, and a lane's channels are read eight shares
+// at a time so that the reads of a channel are in flight together.
 __global__ __launch_bounds__(256) void attn_tile_merge_kernel(const float* __restrict__ part,
                                                               bf16_t* __restrict__ out, int rows, int nsplit,
                                                               int sink, const float* __restrict__ sink_values,
@@ -470,20 +472,31 @@ __global__ __launch_bounds__(256) void attn_tile_merge_kernel(const float* __res
     const int lane = threadIdx.x & (RL_WAVE - 1);
     if (row >= rows) return;
     const float* p = part + (size_t)row * nsplit * (DV + 2);
-    float top = -INFINITY;
-    for (int s = 0; s < nsplit; ++s) top = fmaxf(top, p[s * (DV + 2) + DV]);
+    const bool mine = lane < nsplit;
+    const float m = mine ? p[lane * (DV + 2) + DV] : -INFINITY;
+    const float l = mine ? p[lane * (DV + 2) + DV + 1] : 0.f;
+    float top = m;
+#pragma unroll
+    for (int off = RL_WAVE / 2; off > 0; off >>= 1) top = fmaxf(top, __shfl_xor(top, off));
     // the sink's score: 0, or a number of the row's head (rows are (token, head) pairs)
     const float s0 = (sink && sink_values) ? sink_values[row % nq] * 1.4426950408889634f : 0.f;
     if (sink) top = fmaxf(top, s0);
+    const float weight = mine ? __builtin_amdgcn_exp2f(m - top) : 0.f;
     float den = 0.f;
-    for (int s = 0; s < nsplit; ++s)
-        den += __builtin_amdgcn_exp2f(p[s * (DV + 2) + DV] - top) * p[s * (DV + 2) + DV + 1];
+    for (int s = 0; s < nsplit; ++s) den += __shfl(weight, s) * __shfl(l, s);
     if (sink) den += __builtin_amdgcn_exp2f(s0 - top);
-    for (int c = lane; c < DV; c += RL_WAVE) {
+    for (int c0 = 0; c0 < DV; c0 += RL_WAVE) {
+        const int c = c0 + lane;
+        const bool live = c < DV;
         float sum = 0.f;
-        for (int s = 0; s < nsplit; ++s)
-            sum += __builtin_amdgcn_exp2f(p[s * (DV + 2) + DV] - top) * p[s * (DV + 2) + c];
-        out[(size_t)row * DV + c] = float_to_bf16(sum / den);
+        for (int s8 = 0; s8 < nsplit; s8 += 8) {
+            float v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = (live && s8 + j < nsplit) ? p[(s8 + j) * (DV + 2) + c] : 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) sum += __shfl(weight, (s8 + j) & (RL_WAVE - 1)) * v[j];
+        }
+        if (live) out[(size_t)row * DV + c] = float_to_bf16(sum / den);
     }
 }
 

@@ -338,6 +338,49 @@ __global__ __launch_bounds__(WAVES* RL_WAVE) void head_product_mfma_kernel(
     *reinterpret_cast<Vec4<T>*>(yr) = out;
 }
 
+// Steps of many tokens: one wave a (16 tokens, head) pair.  The wave keeps its tokens' inputs in
+// registers (CH chunks of 16) and walks the head's output tiles, so a token's inputs are read once
+// and the head's matrix comes from the caches, where the waves of a workgroup (64 consecutive
+// tokens of one head) and of its neighbours find it.  Every output's sum runs over the same chunks
+// in the same order as in the kernel above: the same bits.
+template <typename T, int WAVES, int CH>
+__global__ __launch_bounds__(WAVES* RL_WAVE) void head_product_rows_kernel(
+    const T* __restrict__ x, const T* __restrict__ w, T* __restrict__ y, int tokens, int I, int O, int x_row,
+    int x_head, int x_off, int y_row, int y_head, int y_off, const T* __restrict__ gate, int gate_row,
+    int gate_col) {
+    typedef typename Quad<T>::type quad;
+    const int lane = threadIdx.x & (RL_WAVE - 1);
+    const int wave = threadIdx.x / RL_WAVE;
+    const int r16 = lane & 15, g = lane >> 4;
+    const int h = blockIdx.y;
+    const int t0 = 16 * (blockIdx.x * WAVES + wave);
+    if (t0 >= tokens) return;
+    const int t = min(t0 + r16, tokens - 1);
+    const T* xr = x + (size_t)t * x_row + x_off + (size_t)h * x_head + 4 * g;
+    const int chunks = I / 16;
+    quad xs[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+        if (c < chunks) xs[c] = *reinterpret_cast<const quad*>(xr + 16 * c);
+    float f = 1.f;
+    if (gate) f = 1.f / (1.f + expf(-to_float(gate[(size_t)t * gate_row + gate_col + h])));
+    const bool live = t0 + r16 < tokens;
+    T* yr = y + (size_t)t * y_row + y_off + (size_t)h * y_head + 4 * g;
+    for (int o0 = 0; o0 < O; o0 += 16) {
+        const T* wr = w + ((size_t)h * O + o0 + r16) * I + 4 * g;
+        f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+            if (c < chunks) acc = mma(*reinterpret_cast<const quad*>(wr + 16 * c), xs[c], acc);
+        if (live) {
+            Vec4<T> out;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) out.v[i] = from_float<T>(acc[i] * f);
+            *reinterpret_cast<Vec4<T>*>(yr + o0) = out;
+        }
+    }
+}
+
 // any sizes: one thread an output element
 template <typename T>
 __global__ void head_product_kernel(const T* __restrict__ x, const T* __restrict__ w, T* __restrict__ y,
@@ -439,6 +482,27 @@ extern "C" int rl_head_product(const void* x, const void* w, void* y, int tokens
     // the matrix cores read four consecutive elements a lane: every offset a multiple of four
     const bool tiles = I % 16 == 0 && O % 16 == 0 && x_row % 4 == 0 && x_head % 4 == 0 && x_off % 4 == 0 &&
                        y_row % 4 == 0 && y_head % 4 == 0 && y_off % 4 == 0;
+    // from this many tokens on a wave keeps 16 tokens' inputs and walks the outputs: below it the
+    // launch of a tile a wave has more waves than the chip has units to give them
+    if (tiles && tokens >= 256 && I <= 512) {
+        constexpr int WAVES = 4;
+        dim3 grid((tokens + 16 * WAVES - 1) / (16 * WAVES), heads), block(WAVES * RL_WAVE);
+#define RL_HEAD_ROWS(TYPE, CH)                                                                                  \
+    hipLaunchKernelGGL((latent::head_product_rows_kernel<TYPE, WAVES, CH>), grid, block, 0, stream, (const TYPE*)x, \
+                       (const TYPE*)w, (TYPE*)y, tokens, I, O, x_row, x_head, x_off, y_row, y_head, y_off,        \
+                       (const TYPE*)gate, gate_row, gate_col)
+        if (act_type == RL_F32) {
+            if (I <= 128) RL_HEAD_ROWS(float, 8);
+            else if (I <= 256) RL_HEAD_ROWS(float, 16);
+            else RL_HEAD_ROWS(float, 32);
+        } else {
+            if (I <= 128) RL_HEAD_ROWS(bf16_t, 8);
+            else if (I <= 256) RL_HEAD_ROWS(bf16_t, 16);
+            else RL_HEAD_ROWS(bf16_t, 32);
+        }
+#undef RL_HEAD_ROWS
+        return rl_launch_status();
+    }
     if (tiles) {
         constexpr int WAVES = 4;
         const int otiles = O / 16;

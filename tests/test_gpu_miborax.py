@@ -342,10 +342,11 @@ def test_rotated_query_part_behind_the_latent_part(dtype, heads, d, rd, rotating
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("heads,I,O", [(4, 16, 32), (3, 80, 16), (1, 16, 16), (8, 96, 16), (2, 144, 128), (5, 10, 18),
                                        (3, 26, 6), (2, 520, 48)])
-@pytest.mark.parametrize("tokens", [1, 37])
+@pytest.mark.parametrize("tokens", [1, 37, 300])
 def test_one_small_matrix_a_head(dtype, heads, I, O, tokens):
     """Slices of every head of ``x`` through the head's own matrix into slices of every head of
-    ``y``, with and without the sigmoid gate per head."""
+    ``y``, with and without the sigmoid gate per head; few tokens (a wave an output tile) and many
+    (a wave 16 tokens and all outputs of a head) give a token the same bits."""
     ops = _ops()
     x_head, y_head, x_off, y_off = I + 8, O + 12, 4, 8
     x = torch.randn(tokens, x_off + heads * x_head).to(dtype)
