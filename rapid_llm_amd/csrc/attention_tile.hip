@@ -44,8 +44,9 @@ constexpr int DV = RL_VALUE_DIM;
 constexpr int DB = D / 16;   // 16-channel chunks of the first product
 constexpr int VB = DV / 16;  // 16-channel blocks of the output
 // blocks of 16 rows a wave multiplies with every key tile it reads, in a bfloat16 step of
-// portions: as many as the registers hold beside two tiles of operands
-constexpr int PORTION_BLOCKS = (D + DV <= 192) ? 4 : ((D + DV <= 384) ? 2 : 1);
+// portions: as many as the registers hold beside two tiles of operands (two up to 320 + 256
+// channels, where they fill every register of a lane without parking any in scratch memory)
+constexpr int PORTION_BLOCKS = (D + DV <= 192) ? 4 : ((D + DV <= 576) ? 2 : 1);
 constexpr int MAX_STAGED_PAGES = 2048;  // page ids of a tile's keys that are staged in LDS
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));

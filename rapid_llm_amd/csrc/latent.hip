@@ -366,7 +366,12 @@ __global__ __launch_bounds__(WAVES* RL_WAVE) void head_product_rows_kernel(
     if (gate) f = 1.f / (1.f + expf(-to_float(gate[(size_t)t * gate_row + gate_col + h])));
     const bool live = t0 + r16 < tokens;
     T* yr = y + (size_t)t * y_row + y_off + (size_t)h * y_head + 4 * g;
-    for (int o0 = 0; o0 < O; o0 += 16) {
+    // blockIdx.z deals the output tiles to gridDim.z workgroups: more waves in flight where a head
+    // has many outputs (the reads of the matrix wait for the caches)
+    const int per = ((O / 16 + gridDim.z - 1) / gridDim.z) * 16;
+    const int o_end = min(O, (int)(blockIdx.z + 1) * per);
+#pragma unroll 2
+    for (int o0 = blockIdx.z * per; o0 < o_end; o0 += 16) {
         const T* wr = w + ((size_t)h * O + o0 + r16) * I + 4 * g;
         f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -486,7 +491,9 @@ extern "C" int rl_head_product(const void* x, const void* w, void* y, int tokens
     // launch of a tile a wave has more waves than the chip has units to give them
     if (tiles && tokens >= 256 && I <= 512) {
         constexpr int WAVES = 4;
-        dim3 grid((tokens + 16 * WAVES - 1) / (16 * WAVES), heads), block(WAVES * RL_WAVE);
+        const int otiles = O / 16;
+        dim3 grid((tokens + 16 * WAVES - 1) / (16 * WAVES), heads, otiles >= 16 ? 4 : (otiles >= 4 ? 2 : 1));
+        dim3 block(WAVES * RL_WAVE);
 #define RL_HEAD_ROWS(TYPE, CH)                                                                                  \
     hipLaunchKernelGGL((latent::head_product_rows_kernel<TYPE, WAVES, CH>), grid, block, 0, stream, (const TYPE*)x, \
                        (const TYPE*)w, (TYPE*)y, tokens, I, O, x_row, x_head, x_off, y_row, y_head, y_off,        \
