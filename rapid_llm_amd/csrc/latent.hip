@@ -323,7 +323,19 @@ __global__ __launch_bounds__(WAVES* RL_WAVE) void head_product_mfma_kernel(
     const T* wr = w + ((size_t)h * O + o0 + r16) * I + 4 * g;
     f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
     const int chunks = I / 16;
-    for (int c = 0; c < chunks; ++c) {
+    // four chunks' operands are read before their products: the reads are in flight together
+    int c = 0;
+    for (; c + 4 <= chunks; c += 4) {
+        quad a[4], b[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            a[j] = *reinterpret_cast<const quad*>(wr + 16 * (c + j));
+            b[j] = *reinterpret_cast<const quad*>(xr + 16 * (c + j));
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc = mma(a[j], b[j], acc);
+    }
+    for (; c < chunks; ++c) {
         const quad a = *reinterpret_cast<const quad*>(wr + 16 * c);
         const quad b = *reinterpret_cast<const quad*>(xr + 16 * c);
         acc = mma(a, b, acc);
@@ -338,51 +350,71 @@ __global__ __launch_bounds__(WAVES* RL_WAVE) void head_product_mfma_kernel(
     *reinterpret_cast<Vec4<T>*>(yr) = out;
 }
 
-// Steps of many tokens: one wave a (16 tokens, head) pair.  The wave keeps its tokens' inputs in
-// registers (CH chunks of 16) and walks the head's output tiles, so a token's inputs are read once
-// and the head's matrix comes from the caches, where the waves of a workgroup (64 consecutive
-// tokens of one head) and of its neighbours find it.  Every output's sum runs over the same chunks
-// in the same order as in the kernel above: the same bits.
-template <typename T, int WAVES, int CH>
+// Blocks of 16 tokens a wave keeps in registers in a step of many tokens: as many as 64 registers
+// a lane hold of CH chunks of inputs.
+template <typename T, int CH>
+constexpr int head_rows_blocks() {
+    constexpr int regs = CH * (int)sizeof(typename Quad<T>::type) / 4;
+    return regs * 4 <= 64 ? 4 : (regs * 2 <= 64 ? 2 : 1);
+}
+
+// Steps of many tokens: one wave a (TB blocks of 16 tokens, head) pair.  The wave keeps its tokens'
+// inputs in registers (CH chunks of 16 a block) and walks the head's output tiles: a token's inputs
+// are read once, and every read of the head's matrix (16 rows of a few bytes each, which the load
+// path takes one cache line after the other) serves TB blocks of tokens.  Every output's sum runs
+// over the same chunks in the same order as in the kernel above: the same bits.  EXACT: the head
+// has exactly CH chunks of inputs and no read hangs on a comparison.
+template <typename T, int WAVES, int CH, bool EXACT>
 __global__ __launch_bounds__(WAVES* RL_WAVE) void head_product_rows_kernel(
     const T* __restrict__ x, const T* __restrict__ w, T* __restrict__ y, int tokens, int I, int O, int x_row,
     int x_head, int x_off, int y_row, int y_head, int y_off, const T* __restrict__ gate, int gate_row,
     int gate_col) {
     typedef typename Quad<T>::type quad;
+    constexpr int TB = head_rows_blocks<T, CH>();
     const int lane = threadIdx.x & (RL_WAVE - 1);
     const int wave = threadIdx.x / RL_WAVE;
     const int r16 = lane & 15, g = lane >> 4;
     const int h = blockIdx.y;
-    const int t0 = 16 * (blockIdx.x * WAVES + wave);
+    const int t0 = 16 * TB * (blockIdx.x * WAVES + wave);
     if (t0 >= tokens) return;
-    const int t = min(t0 + r16, tokens - 1);
-    const T* xr = x + (size_t)t * x_row + x_off + (size_t)h * x_head + 4 * g;
     const int chunks = I / 16;
-    quad xs[CH];
+    quad xs[TB][CH];
+    float f[TB];
+    int t[TB];
 #pragma unroll
-    for (int c = 0; c < CH; ++c)
-        if (c < chunks) xs[c] = *reinterpret_cast<const quad*>(xr + 16 * c);
-    float f = 1.f;
-    if (gate) f = 1.f / (1.f + expf(-to_float(gate[(size_t)t * gate_row + gate_col + h])));
-    const bool live = t0 + r16 < tokens;
-    T* yr = y + (size_t)t * y_row + y_off + (size_t)h * y_head + 4 * g;
-    // blockIdx.z deals the output tiles to gridDim.z workgroups: more waves in flight where a head
-    // has many outputs (the reads of the matrix wait for the caches)
-    const int per = ((O / 16 + gridDim.z - 1) / gridDim.z) * 16;
-    const int o_end = min(O, (int)(blockIdx.z + 1) * per);
-#pragma unroll 2
-    for (int o0 = blockIdx.z * per; o0 < o_end; o0 += 16) {
-        const T* wr = w + ((size_t)h * O + o0 + r16) * I + 4 * g;
-        f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int b = 0; b < TB; ++b) {
+        t[b] = min(t0 + 16 * b + r16, tokens - 1);
+        const T* xr = x + (size_t)t[b] * x_row + x_off + (size_t)h * x_head + 4 * g;
 #pragma unroll
         for (int c = 0; c < CH; ++c)
-            if (c < chunks) acc = mma(*reinterpret_cast<const quad*>(wr + 16 * c), xs[c], acc);
-        if (live) {
-            Vec4<T> out;
+            if (EXACT || c < chunks) xs[b][c] = *reinterpret_cast<const quad*>(xr + 16 * c);
+        f[b] = 1.f;
+        if (gate) f[b] = 1.f / (1.f + expf(-to_float(gate[(size_t)t[b] * gate_row + gate_col + h])));
+    }
+    // blockIdx.z deals the output tiles to gridDim.z workgroups: more waves in flight where a head
+    // has many outputs
+    const int per = ((O / 16 + gridDim.z - 1) / gridDim.z) * 16;
+    const int o_end = min(O, (int)(blockIdx.z + 1) * per);
+    for (int o0 = blockIdx.z * per; o0 < o_end; o0 += 16) {
+        const T* wr = w + ((size_t)h * O + o0 + r16) * I + 4 * g;
+        f32x4 acc[TB];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) out.v[i] = from_float<T>(acc[i] * f);
-            *reinterpret_cast<Vec4<T>*>(yr + o0) = out;
-        }
+        for (int b = 0; b < TB; ++b) acc[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+            if (EXACT || c < chunks) {
+                const quad a = *reinterpret_cast<const quad*>(wr + 16 * c);
+#pragma unroll
+                for (int b = 0; b < TB; ++b) acc[b] = mma(a, xs[b][c], acc[b]);
+            }
+#pragma unroll
+        for (int b = 0; b < TB; ++b)
+            if (t0 + 16 * b + r16 < tokens) {
+                Vec4<T> out;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) out.v[i] = from_float<T>(acc[b][i] * f[b]);
+                *reinterpret_cast<Vec4<T>*>(y + (size_t)t[b] * y_row + y_off + (size_t)h * y_head + 4 * g + o0) = out;
+            }
     }
 }
 
@@ -492,21 +524,35 @@ extern "C" int rl_head_product(const void* x, const void* w, void* y, int tokens
     if (tiles && tokens >= 256 && I <= 512) {
         constexpr int WAVES = 4;
         const int otiles = O / 16;
-        dim3 grid((tokens + 16 * WAVES - 1) / (16 * WAVES), heads, otiles >= 16 ? 4 : (otiles >= 4 ? 2 : 1));
+        dim3 grid(1, heads, otiles >= 16 ? 4 : (otiles >= 4 ? 2 : 1));
         dim3 block(WAVES * RL_WAVE);
-#define RL_HEAD_ROWS(TYPE, CH)                                                                                  \
-    hipLaunchKernelGGL((latent::head_product_rows_kernel<TYPE, WAVES, CH>), grid, block, 0, stream, (const TYPE*)x, \
-                       (const TYPE*)w, (TYPE*)y, tokens, I, O, x_row, x_head, x_off, y_row, y_head, y_off,        \
-                       (const TYPE*)gate, gate_row, gate_col)
+#define RL_HEAD_ROWS(TYPE, CH, EXACT)                                                                              \
+    do {                                                                                                             \
+        grid.x = (tokens + 16 * WAVES * latent::head_rows_blocks<TYPE, CH>() - 1) /                                    \
+                 (16 * WAVES * latent::head_rows_blocks<TYPE, CH>());                                                  \
+        hipLaunchKernelGGL((latent::head_product_rows_kernel<TYPE, WAVES, CH, EXACT>), grid, block, 0, stream,          \
+                           (const TYPE*)x, (const TYPE*)w, (TYPE*)y, tokens, I, O, x_row, x_head, x_off, y_row, y_head, \
+                           y_off, (const TYPE*)gate, gate_row, gate_col);                                               \
+    } while (0)
+#define RL_HEAD_ROWS_OF(TYPE)                       \
+    switch (I / 16) {                               \
+        case 1: RL_HEAD_ROWS(TYPE, 1, true); break;   \
+        case 2: RL_HEAD_ROWS(TYPE, 2, true); break;   \
+        case 4: RL_HEAD_ROWS(TYPE, 4, true); break;   \
+        case 8: RL_HEAD_ROWS(TYPE, 8, true); break;   \
+        case 16: RL_HEAD_ROWS(TYPE, 16, true); break; \
+        case 32: RL_HEAD_ROWS(TYPE, 32, true); break; \
+        default:                                    \
+            if (I <= 128) RL_HEAD_ROWS(TYPE, 8, false);       \
+            else if (I <= 256) RL_HEAD_ROWS(TYPE, 16, false); \
+            else RL_HEAD_ROWS(TYPE, 32, false);               \
+    }
         if (act_type == RL_F32) {
-            if (I <= 128) RL_HEAD_ROWS(float, 8);
-            else if (I <= 256) RL_HEAD_ROWS(float, 16);
-            else RL_HEAD_ROWS(float, 32);
+            RL_HEAD_ROWS_OF(float)
         } else {
-            if (I <= 128) RL_HEAD_ROWS(bf16_t, 8);
-            else if (I <= 256) RL_HEAD_ROWS(bf16_t, 16);
-            else RL_HEAD_ROWS(bf16_t, 32);
+            RL_HEAD_ROWS_OF(bf16_t)
         }
+#undef RL_HEAD_ROWS_OF
 #undef RL_HEAD_ROWS
         return rl_launch_status();
     }

@@ -341,7 +341,8 @@ def test_rotated_query_part_behind_the_latent_part(dtype, heads, d, rd, rotating
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("heads,I,O", [(4, 16, 32), (3, 80, 16), (1, 16, 16), (8, 96, 16), (2, 144, 128), (5, 10, 18),
-                                       (3, 26, 6), (2, 520, 48)])
+                                       (3, 26, 6), (2, 520, 48), (2, 128, 80), (3, 256, 32), (1, 512, 16), (2, 32, 272),
+                                       (2, 64, 64)])
 @pytest.mark.parametrize("tokens", [1, 37, 300])
 def test_one_small_matrix_a_head(dtype, heads, I, O, tokens):
     """Slices of every head of ``x`` through the head's own matrix into slices of every head of
