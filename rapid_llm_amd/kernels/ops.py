@@ -1476,8 +1476,17 @@ def attention_tile(
     # a bfloat16 step with portions: tiles of several blocks of 16 rows, so that the keys a
     # workgroup reads serve more rows (float32 keeps one order of summation, whatever the step)
     tile_rows = 16
-    if q.dtype == torch.bfloat16 and max(ctx.h_seq_lens) * group > 16:
+    longest = max(ctx.h_seq_lens)
+    if q.dtype == torch.bfloat16 and longest * group > 16:
         tile_rows = lib.rl_attn_tile_wide_rows()
+        if longest == 1 and tile_rows > 16:
+            # single tokens whose heads fill several blocks of rows: where the keys are many,
+            # dealing them to several workgroups is worth more than sharing a key tile between
+            # the blocks of one
+            blocks = len(ctx.h_seq_lens) * -(-group // 16) * nkv
+            bound = _static(ctx).get("context_bound", ctx.max_position + 1)
+            if tile_splits(blocks, bound, window, keep_first) > 1:
+                tile_rows = 16
     tiles, num_tiles = _f32_tiles(ctx, group, tile_rows)
     # few tiles over many keys (a step of single tokens, mostly): a tile's keys are dealt to
     # several workgroups, on compute units of their own, and their shares merged

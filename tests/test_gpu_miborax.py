@@ -132,6 +132,9 @@ ATTENTION_CASES = [
     (3, 36, 26, 8, 0, [(0, 40), (9, 1), (10, 1), (130, 2)]),
     (2, 24, 18, 8, 9, [(0, 30), (8, 1), (9, 1), (10, 1)]),
     (2, 64, 32, 4, 0, [(8300, 1), (8250, 60)]),  # more pages than a workgroup stages: the table is read
+    (32, 64, 32, 16, 0, [(3000, 1), (1500, 1), (40, 1)]),  # more heads than a block of rows holds: single tokens far in,
+    (32, 64, 32, 16, 0, [(40, 1), (7, 1)]),                # near the start,
+    (20, 32, 16, 8, 19, [(45, 1), (0, 30), (200, 3)]),     # and a last block that is not full, beside portions
 ]
 
 
