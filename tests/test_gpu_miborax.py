@@ -128,6 +128,7 @@ ATTENTION_CASES = [
     (4, 128, 96, 16, 64, [(0, 140), (63, 1), (64, 1), (65, 1), (1000, 1)]),
     (2, 160, 144, 16, 130, [(0, 200), (129, 1), (130, 1), (131, 1)]),
     (3, 320, 256, 16, 50, [(0, 70), (49, 1), (50, 1), (400, 1)]),      # rows wider than a lane's registers were sized for
+    (2, 576, 512, 16, 0, [(0, 40), (100, 1), (300, 2)]),               # the widest rows the kernel is built for
     (5, 24, 18, 8, 33, [(0, 50), (32, 1), (33, 1), (100, 1)]),         # sizes off the grid of 16
     (3, 36, 26, 8, 0, [(0, 40), (9, 1), (10, 1), (130, 2)]),
     (2, 24, 18, 8, 9, [(0, 30), (8, 1), (9, 1), (10, 1)]),
