@@ -305,7 +305,9 @@ struct Quad<bf16_t> {
 // (o, g) holds inputs 4g .. 4g + 3 of its output row), the tokens the second (lane (t, g) the
 // same inputs of its token), and a lane ends with outputs 4g .. 4g + 3 of its own token.  The sum
 // over the inputs runs in ascending chunks of 16 whatever the step holds.
-template <typename T, int WAVES>
+// CH > 0: the head has exactly CH chunks of inputs, and all of a tile's operands are read before
+// the first product (a step of a few tokens is all latency here); CH 0: any number of chunks.
+template <typename T, int WAVES, int CH>
 __global__ __launch_bounds__(WAVES* RL_WAVE) void head_product_mfma_kernel(
     const T* __restrict__ x, const T* __restrict__ w, T* __restrict__ y, int tokens, int I, int O, int x_row,
     int x_head, int x_off, int y_row, int y_head, int y_off, const T* __restrict__ gate, int gate_row,
@@ -323,8 +325,19 @@ __global__ __launch_bounds__(WAVES* RL_WAVE) void head_product_mfma_kernel(
     const T* wr = w + ((size_t)h * O + o0 + r16) * I + 4 * g;
     f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
     const int chunks = I / 16;
-    // four chunks' operands are read before their products: the reads are in flight together
     int c = 0;
+    if (CH > 0) {
+        quad a[CH > 0 ? CH : 1], b[CH > 0 ? CH : 1];
+#pragma unroll
+        for (int j = 0; j < CH; ++j) {
+            a[j] = *reinterpret_cast<const quad*>(wr + 16 * j);
+            b[j] = *reinterpret_cast<const quad*>(xr + 16 * j);
+        }
+#pragma unroll
+        for (int j = 0; j < CH; ++j) acc = mma(a[j], b[j], acc);
+        c = chunks;
+    }
+    // four chunks' operands are read before their products: the reads are in flight together
     for (; c + 4 <= chunks; c += 4) {
         quad a[4], b[4];
 #pragma unroll
@@ -561,14 +574,26 @@ extern "C" int rl_head_product(const void* x, const void* w, void* y, int tokens
         const int otiles = O / 16;
         dim3 grid((tokens + 15) / 16, heads, (otiles + WAVES - 1) / WAVES), block(WAVES * RL_WAVE);
         if (grid.z > 65535) return RL_ERR_ARG;
-        if (act_type == RL_F32)
-            hipLaunchKernelGGL((latent::head_product_mfma_kernel<float, WAVES>), grid, block, 0, stream,
-                               (const float*)x, (const float*)w, (float*)y, tokens, I, O, x_row, x_head, x_off,
-                               y_row, y_head, y_off, (const float*)gate, gate_row, gate_col);
-        else
-            hipLaunchKernelGGL((latent::head_product_mfma_kernel<bf16_t, WAVES>), grid, block, 0, stream,
-                               (const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, tokens, I, O, x_row, x_head, x_off,
-                               y_row, y_head, y_off, (const bf16_t*)gate, gate_row, gate_col);
+#define RL_HEAD_TILE(TYPE, CH)                                                                                    \
+    hipLaunchKernelGGL((latent::head_product_mfma_kernel<TYPE, WAVES, CH>), grid, block, 0, stream, (const TYPE*)x, \
+                       (const TYPE*)w, (TYPE*)y, tokens, I, O, x_row, x_head, x_off, y_row, y_head, y_off,          \
+                       (const TYPE*)gate, gate_row, gate_col)
+#define RL_HEAD_TILE_OF(TYPE)                  \
+    switch (I / 16) {                          \
+        case 1: RL_HEAD_TILE(TYPE, 1); break;   \
+        case 2: RL_HEAD_TILE(TYPE, 2); break;   \
+        case 4: RL_HEAD_TILE(TYPE, 4); break;   \
+        case 8: RL_HEAD_TILE(TYPE, 8); break;   \
+        case 16: RL_HEAD_TILE(TYPE, 16); break; \
+        default: RL_HEAD_TILE(TYPE, 0);         \
+    }
+        if (act_type == RL_F32) {
+            RL_HEAD_TILE_OF(float)
+        } else {
+            RL_HEAD_TILE_OF(bf16_t)
+        }
+#undef RL_HEAD_TILE_OF
+#undef RL_HEAD_TILE
         return rl_launch_status();
     }
     const size_t total = (size_t)tokens * heads * O;
