@@ -41,6 +41,8 @@ _LAZY: dict[str, str] = {
     "sikevik": "rapid_llm_amd.models.sikevik",
     "Miborax": "rapid_llm_amd.models.miborax",
     "miborax": "rapid_llm_amd.models.miborax",
+    "Fomunex": "rapid_llm_amd.models.fomunex",
+    "fomunex": "rapid_llm_amd.models.fomunex",
 }
 
 

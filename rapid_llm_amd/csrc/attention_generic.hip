@@ -6,7 +6,9 @@
 // (window 0: all keys), which were written before this kernel runs.  With a window, the first
 // keep_first keys of the request are read as well; a value head has dv channels, which need not
 // be d; with `sink` the softmax's denominator has one more term, exp(0) or, with `sink_values`,
-// exp of a number per query head: a key without a value.
+// exp of a number per query head: a key without a value.  With cap > 0 a scaled score s becomes
+// cap * tanh(s / cap); with `slopes` (one number a query head) slope_h * (pos - j) is then taken
+// off it.
 //
 // Scores (q . k) / sqrt(d) (rapid_llm/modules/attention.py:62), online softmax over tiles
 // of 256 keys in ascending order (rapid_llm/kernels/ops/attention/flashattention2_nopad.py:
@@ -21,7 +23,8 @@ __global__ __launch_bounds__(ATT_THREADS) void attention_generic_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     T* __restrict__ out, const int* __restrict__ positions, const int* __restrict__ token_slot,
     const int* __restrict__ block_table, int table_stride, int page_size, int nq, int nkv, int d,
-    int window, float scale, int dv, int keep_first, int sink, const float* __restrict__ sink_values) {
+    int window, float scale, int dv, int keep_first, int sink, const float* __restrict__ sink_values,
+    float cap, const float* __restrict__ slopes) {
     __shared__ float qs[256];
     __shared__ float ps[ATT_THREADS];
     __shared__ int key_page[ATT_THREADS];  // page * nkv + kv head of each key of the tile
@@ -58,6 +61,8 @@ __global__ __launch_bounds__(ATT_THREADS) void attention_generic_kernel(
             float dot = 0.f;
             for (int i = 0; i < d; ++i) dot = fmaf(qs[i], to_float(krow[i]), dot);
             s = dot * scale;
+            if (cap > 0.f) s = cap * tanhf(s / cap);
+            if (slopes) s -= slopes[h] * (float)(pos - j);
         }
         const float tile_max = block_max(s, scratch);  // finite: the tile holds >= 1 key
         const float m_new = fmaxf(m, tile_max);
@@ -93,9 +98,10 @@ extern "C" int rl_attention_generic(const void* q, const void* k_cache, const vo
                                     void* out, const int* positions, const int* token_slot,
                                     const int* block_table, int table_stride, int page_size,
                                     int tokens, int nq, int nkv, int d, int window, float scale,
-                                    int dv, int keep_first, int sink, const float* sink_values, int act_type,
-                                    hipStream_t stream) {
+                                    int dv, int keep_first, int sink, const float* sink_values, float cap,
+                                    const float* slopes, int act_type, hipStream_t stream) {
     if (tokens <= 0) return RL_OK;
+    if (cap < 0.f) return RL_ERR_ARG;
     if (d < 1 || d > 256 || dv < 1 || dv > 256 || keep_first < 0 || nkv < 1 || nq % nkv || page_size < 1 ||
         nq > 65535)
         return RL_ERR_ARG;
@@ -104,12 +110,12 @@ extern "C" int rl_attention_generic(const void* q, const void* k_cache, const vo
         hipLaunchKernelGGL(attention_generic_kernel<float>, grid, block, 0, stream,
                            (const float*)q, (const float*)k_cache, (const float*)v_cache,
                            (float*)out, positions, token_slot, block_table, table_stride,
-                           page_size, nq, nkv, d, window, scale, dv, keep_first, sink, sink_values);
+                           page_size, nq, nkv, d, window, scale, dv, keep_first, sink, sink_values, cap, slopes);
     else if (act_type == RL_BF16)
         hipLaunchKernelGGL(attention_generic_kernel<bf16_t>, grid, block, 0, stream,
                            (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
                            (bf16_t*)out, positions, token_slot, block_table, table_stride,
-                           page_size, nq, nkv, d, window, scale, dv, keep_first, sink, sink_values);
+                           page_size, nq, nkv, d, window, scale, dv, keep_first, sink, sink_values, cap, slopes);
     else
         return RL_ERR_ARG;
     return rl_launch_status();

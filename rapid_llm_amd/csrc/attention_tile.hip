@@ -21,6 +21,10 @@
 // the window of the tile's first row up to its last row's position.  With `sink` the softmax's
 // denominator is 1 + sum_j exp(s_j): a key of score 0 that carries no value.
 //
+// Two options change a score s = (q . k) scale before the softmax: with cap > 0 it becomes
+// cap * tanh(s / cap), and with `slopes` (one number a query head) slope_h * (p - j) is taken off
+// it afterwards.  The sink's term has neither.
+//
 // A row's result does not depend on the tile it falls in, on the other rows there, or on how a
 // prompt was cut into steps: keys are taken in tiles of 16 at absolute positions 0, 16, ..,
 // each wave takes its tiles in ascending order; within a tile the order of every sum is fixed
@@ -108,6 +112,18 @@ template <>
 __device__ inline float fexp<bf16_t>(float x) {
     return __builtin_amdgcn_exp2f(x);
 }
+// tanh of a capped score: the library's in float32; in bfloat16 1 - 2 / (1 + e^(2x)) on the
+// hardware's exponential and reciprocal (exact at both ends: e^(2x) = inf gives 1, 0 gives -1)
+template <typename T>
+__device__ inline float ftanh(float x);
+template <>
+__device__ inline float ftanh<float>(float x) {
+    return tanhf(x);
+}
+template <>
+__device__ inline float ftanh<bf16_t>(float x) {
+    return 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(2.8853900817779268f * x));
+}
 
 // the four lanes (r, g = 0..3) that share a row: the same bits in each of them.  Two lane swaps
 // of gfx950 (the halves of the wave, then neighbouring rows of 16) instead of two trips through
@@ -138,9 +154,14 @@ __global__ __launch_bounds__(AW* RL_WAVE) void attn_tile_kernel(
     T* __restrict__ out, const int* __restrict__ tile_info, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
     int page_size, int nq, int nkv, int window, int keep_first, int sink, float scale,
-    float* __restrict__ part, int nsplit, const float* __restrict__ sink_values) {
+    float* __restrict__ part, int nsplit, const float* __restrict__ sink_values, float cap,
+    const float* __restrict__ slopes) {
     typedef typename Quad<T>::type quad;
-    if constexpr (sizeof(T) == 2) scale *= 1.4426950408889634f;  // scores in units of log2
+    const float in_log2 = sizeof(T) == 2 ? 1.4426950408889634f : 1.f;  // bfloat16: scores in units of log2
+    const float cap_in = cap > 0.f ? scale / cap : 0.f;  // a raw product times this is s / cap
+    const float cap_out = cap * in_log2;
+    const bool adjusted = cap > 0.f || slopes != nullptr;
+    scale *= in_log2;
     const int tile = blockIdx.x;
     const int hk = blockIdx.y;
     const int G = nq / nkv;
@@ -168,6 +189,15 @@ __global__ __launch_bounds__(AW* RL_WAVE) void attn_tile_kernel(
         kend[r] = pos + 1;
         kstart[r] = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
     }
+    float slope[R];  // what a position of distance costs this lane's row, in the scores' unit
+#pragma unroll
+    for (int r = 0; r < R; ++r) slope[r] = slopes ? slopes[head[r]] * in_log2 : 0.f;
+    // a raw product of row r and key `key` as the softmax takes it
+    auto scored = [&](float raw, int key, int r) -> float {
+        if (!adjusted) return raw * scale;
+        const float v = cap > 0.f ? cap_out * ftanh<T>(raw * cap_in) : raw * scale;
+        return v - slope[r] * (float)(kend[r] - 1 - key);
+    };
     const int blocks = min(R, (rows - row0 + 15) / 16);  // blocks of the tile that hold rows
     // keys [all_lo, all_hi) are seen by every row of a block (none where the block is not full):
     // a tile of keys inside needs no masks
@@ -272,7 +302,7 @@ __global__ __launch_bounds__(AW* RL_WAVE) void attn_tile_kernel(
         if (kb >= all_lo[r] && kb + 16 <= all_hi[r]) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                s[i] *= scale;
+                s[i] = scored(s[i], kb + 4 * g + i, r);
                 tmax = fmaxf(tmax, s[i]);
             }
         } else {
@@ -280,7 +310,7 @@ __global__ __launch_bounds__(AW* RL_WAVE) void attn_tile_kernel(
             for (int i = 0; i < 4; ++i) {
                 const int key = kb + 4 * g + i;
                 const bool seen = row_ok[r] && key < kend[r] && (key >= kstart[r] || key < keep);
-                s[i] = seen ? s[i] * scale : -INFINITY;
+                s[i] = seen ? scored(s[i], key, r) : -INFINITY;
                 tmax = fmaxf(tmax, s[i]);
             }
         }
@@ -519,8 +549,9 @@ extern "C" int rl_attn_tile(const void* q, const void* k_cache, const void* v_ca
                             const int* token_slot, const int* block_table, int table_stride,
                             int page_size, int nq, int nkv, int window, int keep_first, int sink,
                             float scale, int nsplit, float* part, int tokens, int tile_rows, int act_type,
-                            const float* sink_values, hipStream_t stream) {
+                            const float* sink_values, float cap, const float* slopes, hipStream_t stream) {
     if (num_tiles <= 0) return RL_OK;
+    if (cap < 0.f) return RL_ERR_ARG;
     if (nkv < 1 || nq % nkv || page_size < 4 || page_size % 4 || nkv > 65535 || window < 0 || keep_first < 0)
         return RL_ERR_ARG;
     constexpr int AW = 4;
@@ -532,7 +563,7 @@ extern "C" int rl_attn_tile(const void* q, const void* k_cache, const void* v_ca
     if (act_type == RL_BF16 && tile_rows == 16 * PB && PB > 1) {
         if (nsplit != 1) return RL_ERR_ARG;
         hipLaunchKernelGGL((tileattn::attn_tile_kernel<bf16_t, AW, PB>), grid, block, 0, stream, RL_TILE_ARGS(bf16_t),
-                           nullptr, 1, sink_values);
+                           nullptr, 1, sink_values, cap, slopes);
         return rl_launch_status();
     }
     if (tile_rows != 16) return RL_ERR_ARG;
@@ -542,7 +573,7 @@ extern "C" int rl_attn_tile(const void* q, const void* k_cache, const void* v_ca
     if (nsplit > 1) {
         if (act_type != RL_BF16 || !part || nsplit > 64 || tokens < 1) return RL_ERR_ARG;
         hipLaunchKernelGGL((tileattn::attn_tile_kernel<bf16_t, AW, 1>), dim3(num_tiles, nkv, nsplit), block, 0, stream,
-                           RL_TILE_ARGS(bf16_t), part, nsplit, sink_values);
+                           RL_TILE_ARGS(bf16_t), part, nsplit, sink_values, cap, slopes);
         const int rows = tokens * nq;
         hipLaunchKernelGGL(tileattn::attn_tile_merge_kernel, dim3((rows + 3) / 4), dim3(256), 0, stream, part,
                            (bf16_t*)out, rows, nsplit, sink, sink_values, nq);
@@ -550,10 +581,10 @@ extern "C" int rl_attn_tile(const void* q, const void* k_cache, const void* v_ca
     }
     if (act_type == RL_F32)
         hipLaunchKernelGGL((tileattn::attn_tile_kernel<float, AW, 1>), grid, block, 0, stream, RL_TILE_ARGS(float),
-                           nullptr, 1, sink_values);
+                           nullptr, 1, sink_values, cap, slopes);
     else if (act_type == RL_BF16)
         hipLaunchKernelGGL((tileattn::attn_tile_kernel<bf16_t, AW, 1>), grid, block, 0, stream, RL_TILE_ARGS(bf16_t),
-                           nullptr, 1, sink_values);
+                           nullptr, 1, sink_values, cap, slopes);
     else
         return RL_ERR_ARG;
 #undef RL_TILE_ARGS

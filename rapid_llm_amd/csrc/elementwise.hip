@@ -9,6 +9,7 @@
 // With `inv_freq` (hidden / 2 float32 frequencies) a sinusoidal position vector is added:
 // channel 2i gets sin(a), channel 2i + 1 cos(a), a = positions[t] * inv_freq[i] as a float32
 // product; sine and cosine of that angle are evaluated in double.
+// With `pos_table` (rows of the table's type, one a position) row positions[t] is added, unscaled.
 // --------------------------------------------------------------------------- //
 __device__ inline float sinusoid_channel(int pos, int channel, const float* __restrict__ inv_freq) {
     const float angle = (float)pos * inv_freq[channel >> 1];
@@ -22,9 +23,10 @@ template <typename W>
 __global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict__ fed, int fed_rows,
                              const W* __restrict__ table, float* __restrict__ out, int hidden,
                              int vocab, float scale, const int* __restrict__ positions,
-                             const float* __restrict__ inv_freq) {
+                             const float* __restrict__ inv_freq, const W* __restrict__ pos_table) {
     const int t = blockIdx.x;
-    const int pos = inv_freq ? positions[t] : 0;
+    const int pos = (inv_freq || pos_table) ? positions[t] : 0;
+    const W* prow = pos_table ? pos_table + (size_t)pos * hidden : nullptr;
     int id = ids[t];
     if (id < 0 && fed && -id - 1 < fed_rows) id = fed[-id - 1];
     // ids are validated on the host; an id outside the table reads row 0 rather than faulting
@@ -38,10 +40,18 @@ __global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict_
         };
         for (int i = threadIdx.x * VEC; i < hidden; i += blockDim.x * VEC) {
             const Pack p = *reinterpret_cast<const Pack*>(row + i);
+            Pack pp;
+            if (prow) pp = *reinterpret_cast<const Pack*>(prow + i);
 #pragma unroll
             for (int j = 0; j < VEC; j += 4) {
                 float4 v = make_float4(to_float(p.v[j]) * scale, to_float(p.v[j + 1]) * scale,
                                        to_float(p.v[j + 2]) * scale, to_float(p.v[j + 3]) * scale);
+                if (prow) {
+                    v.x += to_float(pp.v[j]);
+                    v.y += to_float(pp.v[j + 1]);
+                    v.z += to_float(pp.v[j + 2]);
+                    v.w += to_float(pp.v[j + 3]);
+                }
                 if (inv_freq) {
                     v.x += sinusoid_channel(pos, i + j, inv_freq);
                     v.y += sinusoid_channel(pos, i + j + 1, inv_freq);
@@ -55,6 +65,7 @@ __global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict_
     }
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
         float v = to_float(row[i]) * scale;
+        if (prow) v += to_float(prow[i]);
         if (inv_freq) v += sinusoid_channel(pos, i, inv_freq);
         dst[i] = v;
     }
@@ -62,16 +73,18 @@ __global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict_
 
 extern "C" int rl_embed(const int* ids, const int* fed, int fed_rows, const void* table,
                         int table_type, float* out, int tokens, int hidden, int vocab, float scale,
-                        const int* positions, const float* inv_freq, hipStream_t stream) {
+                        const int* positions, const float* inv_freq, const void* pos_table, hipStream_t stream) {
     if (tokens <= 0) return RL_OK;
-    if (inv_freq && !positions) return RL_ERR_ARG;
+    if ((inv_freq || pos_table) && !positions) return RL_ERR_ARG;
     dim3 grid(tokens), block(256);
     if (table_type == RL_F32)
         hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, ids, fed, fed_rows,
-                           (const float*)table, out, hidden, vocab, scale, positions, inv_freq);
+                           (const float*)table, out, hidden, vocab, scale, positions, inv_freq,
+                           (const float*)pos_table);
     else if (table_type == RL_BF16)
         hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, ids, fed, fed_rows,
-                           (const bf16_t*)table, out, hidden, vocab, scale, positions, inv_freq);
+                           (const bf16_t*)table, out, hidden, vocab, scale, positions, inv_freq,
+                           (const bf16_t*)pos_table);
     else
         return RL_ERR_ARG;
     return rl_launch_status();
@@ -514,12 +527,14 @@ extern "C" int rl_add_rmsnorm_parts(float* residual, const float* parts, int npa
 // limit > 0: the clamped variant, g' = min(g, limit), u' = clamp(u, -limit, limit),
 // g' * sigmoid(alpha * g') * (u' + 1).
 // With `route` (float32 [tokens, experts]) the first experts * ff hidden units of a row are those
-// of `experts` experts side by side, and expert e's are multiplied by route[t, e].
+// of `experts` experts side by side, and expert e's are multiplied by route[t, e]; with
+// `route_input` the gate and up values are multiplied by it instead, before the activation (an
+// expert whose input was scaled: its two products are linear).
 // --------------------------------------------------------------------------- //
 template <typename T>
 __global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inter,
                               size_t total, float limit, float alpha, const float* __restrict__ route,
-                              int experts, int ff) {
+                              int experts, int ff, int route_input) {
     size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t step = (size_t)gridDim.x * blockDim.x;
     for (; idx < total; idx += step) {
@@ -528,8 +543,9 @@ __global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out
         const T* row = gate_up + t * 2 * (size_t)inter;
         const float g = to_float(row[j]);
         const float u = to_float(row[inter + j]);
-        float v = glu_act(g, u, limit, alpha);
-        if (route && j < experts * ff) v *= route[t * experts + j / ff];
+        const float factor = (route && j < experts * ff) ? route[t * experts + j / ff] : 1.f;
+        const float v = route_input ? glu_act(g * factor, u * factor, limit, alpha)
+                                    : glu_act(g, u, limit, alpha) * factor;
         out[idx] = from_float<T>(v);
     }
 }
@@ -543,7 +559,7 @@ struct alignas(sizeof(T) * 8) Vec8 {
 template <typename T>
 __global__ void swiglu_vec_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inter,
                                   size_t total_vec, float limit, float alpha, const float* __restrict__ route,
-                                  int experts, int ff) {
+                                  int experts, int ff, int route_input) {
     size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t step = (size_t)gridDim.x * blockDim.x;
     const int per_row = inter >> 3;
@@ -558,7 +574,9 @@ __global__ void swiglu_vec_kernel(const T* __restrict__ gate_up, T* __restrict__
         Vec8<T> y;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            y.v[i] = from_float<T>(glu_act(to_float(g.v[i]), to_float(u.v[i]), limit, alpha) * factor);
+            y.v[i] = from_float<T>(
+                route_input ? glu_act(to_float(g.v[i]) * factor, to_float(u.v[i]) * factor, limit, alpha)
+                            : glu_act(to_float(g.v[i]), to_float(u.v[i]), limit, alpha) * factor);
         }
         *reinterpret_cast<Vec8<T>*>(out + t * (size_t)inter + j) = y;
     }
@@ -566,31 +584,34 @@ __global__ void swiglu_vec_kernel(const T* __restrict__ gate_up, T* __restrict__
 
 template <typename T>
 static void launch_swiglu(const T* gate_up, T* out, int tokens, int inter, float limit, float alpha,
-                          const float* route, int experts, int ff, hipStream_t stream) {
+                          const float* route, int experts, int ff, int route_input, hipStream_t stream) {
     if (inter % 8 == 0 && (!route || ff % 8 == 0)) {
         const size_t total = (size_t)tokens * (inter / 8);
         size_t blocks = (total + 255) / 256;
         if (blocks > 65536) blocks = 65536;
         hipLaunchKernelGGL(swiglu_vec_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream,
-                           gate_up, out, inter, total, limit, alpha, route, experts, ff);
+                           gate_up, out, inter, total, limit, alpha, route, experts, ff, route_input);
         return;
     }
     const size_t total = (size_t)tokens * inter;
     size_t blocks = (total + 255) / 256;
     if (blocks > 65536) blocks = 65536;
     hipLaunchKernelGGL(swiglu_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, gate_up, out,
-                       inter, total, limit, alpha, route, experts, ff);
+                       inter, total, limit, alpha, route, experts, ff, route_input);
 }
 
 extern "C" int rl_swiglu(const void* gate_up, void* out, int tokens, int inter, int act_type,
-                         float limit, float alpha, const float* route, int experts, int ff, hipStream_t stream) {
+                         float limit, float alpha, const float* route, int experts, int ff, int route_input,
+                         hipStream_t stream) {
     if (tokens <= 0) return RL_OK;
     if (route && (experts < 1 || ff < 1 || (long)experts * ff > inter)) return RL_ERR_ARG;
+    if (route_input && !route) return RL_ERR_ARG;
     if (act_type == RL_F32)
-        launch_swiglu<float>((const float*)gate_up, (float*)out, tokens, inter, limit, alpha, route, experts, ff, stream);
+        launch_swiglu<float>((const float*)gate_up, (float*)out, tokens, inter, limit, alpha, route, experts, ff,
+                             route_input, stream);
     else if (act_type == RL_BF16)
         launch_swiglu<bf16_t>((const bf16_t*)gate_up, (bf16_t*)out, tokens, inter, limit, alpha, route, experts,
-                              ff, stream);
+                              ff, route_input, stream);
     else
         return RL_ERR_ARG;
     return rl_launch_status();
@@ -600,6 +621,7 @@ extern "C" int rl_swiglu(const void* gate_up, void* out, int tokens, int inter, 
 // One-operand activations of a two-layer feed-forward, out = act(x):
 //   kind 0: gelu in its tanh form, 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))
 //   kind 1: relu(z)^2
+//   kind 2: tanh(z)
 // With `route` (float32 [tokens, experts]) the first experts * ff columns of a row are the
 // hidden units of `experts` experts side by side, and expert e's units are multiplied by
 // route[t, e] (0 for an expert the token does not use); columns beyond (a shared expert's)
@@ -610,6 +632,7 @@ __device__ inline float unary_act(float z, int kind) {
         const float r = fmaxf(z, 0.f);
         return r * r;
     }
+    if (kind == 2) return tanhf(z);
     return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
 
@@ -657,7 +680,7 @@ __global__ void unary_act_vec_kernel(const T* __restrict__ x, T* __restrict__ ou
 extern "C" int rl_unary_act(const void* x, void* out, int tokens, int cols, int kind, const float* route,
                             int experts, int ff, int act_type, hipStream_t stream) {
     if (tokens <= 0 || cols <= 0) return RL_OK;
-    if (kind < 0 || kind > 1) return RL_ERR_ARG;
+    if (kind < 0 || kind > 2) return RL_ERR_ARG;
     if (route && (experts < 1 || ff < 1 || (long)experts * ff > cols)) return RL_ERR_ARG;
     if (act_type != RL_F32 && act_type != RL_BF16) return RL_ERR_ARG;
     const bool vec = cols % 8 == 0 && (!route || ff % 8 == 0);
@@ -685,10 +708,36 @@ extern "C" int rl_unary_act(const void* x, void* out, int tokens, int cols, int 
 //   s = softmax(z) over all experts; the `top` largest are chosen (the lower index wins a tie);
 //   route[t, e] = s_e / (sum of the chosen s + 1e-20) * scale for a chosen expert, else 0.
 // z is overwritten by route.
+// With `sigmoid` scores, s = 1 / (1 + exp(-z)) and a chosen expert's weight is s_e * scale as it
+// is: the chosen scores are not divided by their sum.
 // --------------------------------------------------------------------------- //
 #define ROUTE_MAX_EXPERTS 1024
 // (a chosen expert's score is marked by its sign: scores are exponentials, never below +0)
-__device__ inline void route_row(float* __restrict__ row, float* __restrict__ dst, int experts, int top, float scale) {
+__device__ inline void route_row(float* __restrict__ row, float* __restrict__ dst, int experts, int top, float scale,
+                                 int sigmoid = 0) {
+    if (sigmoid) {
+        // the largest logits are the largest scores; a chosen one is marked by a NaN-free trick:
+        // its score, a number in (0, 1), is stored negated
+        for (int e = 0; e < experts; ++e) row[e] = 1.f / (1.f + expf(-row[e]));
+        for (int k = 0; k < top; ++k) {
+            int best = -1;
+            float best_s = -1.f;
+            for (int e = 0; e < experts; ++e) {
+                const float p = row[e];
+                if (!signbit(p) && p > best_s) {
+                    best_s = p;
+                    best = e;
+                }
+            }
+            if (best < 0) break;
+            row[best] = -best_s;  // -0.f for a score that underflowed: still marked by its sign
+        }
+        for (int e = 0; e < experts; ++e) {
+            const float p = row[e];
+            dst[e] = signbit(p) ? -p * scale : 0.f;
+        }
+        return;
+    }
     float m = -INFINITY;
     for (int e = 0; e < experts; ++e) m = fmaxf(m, row[e]);
     float total = 0.f;
@@ -739,7 +788,8 @@ extern "C" int rl_route(float* z, int tokens, int experts, int top, float scale,
 template <typename T>
 __global__ __launch_bounds__(256) void router_kernel(const T* __restrict__ x, const float* __restrict__ w,
                                                      float* __restrict__ route, int tokens, int k, int experts,
-                                                     int top, float scale, const float* __restrict__ bias) {
+                                                     int top, float scale, const float* __restrict__ bias,
+                                                     int sigmoid) {
     extern __shared__ float s_logits[];  // [4][experts]
     const int lane = threadIdx.x & (RL_WAVE - 1);
     const int wave = threadIdx.x / RL_WAVE;
@@ -783,21 +833,21 @@ __global__ __launch_bounds__(256) void router_kernel(const T* __restrict__ x, co
             if (lane == 0 && j < ne) z[e0 + j] = bias ? sum + bias[e0 + j] : sum;
         }
     }
-    if (lane == 0) route_row(z, route + (size_t)t * experts, experts, top, scale);
+    if (lane == 0) route_row(z, route + (size_t)t * experts, experts, top, scale, sigmoid);
 }
 
 extern "C" int rl_router(const void* x, const float* w, float* route, int tokens, int k, int experts, int top,
-                         float scale, const float* bias, int act_type, hipStream_t stream) {
+                         float scale, const float* bias, int sigmoid, int act_type, hipStream_t stream) {
     if (tokens <= 0) return RL_OK;
     if (k < 1 || experts < 1 || experts > ROUTE_MAX_EXPERTS || top < 1 || top > experts) return RL_ERR_ARG;
     dim3 grid((tokens + 3) / 4), block(256);
     const size_t lds = (size_t)4 * experts * sizeof(float);
     if (act_type == RL_F32)
         hipLaunchKernelGGL(router_kernel<float>, grid, block, lds, stream, (const float*)x, w, route, tokens, k,
-                           experts, top, scale, bias);
+                           experts, top, scale, bias, sigmoid);
     else if (act_type == RL_BF16)
         hipLaunchKernelGGL(router_kernel<bf16_t>, grid, block, lds, stream, (const bf16_t*)x, w, route, tokens, k,
-                           experts, top, scale, bias);
+                           experts, top, scale, bias, sigmoid);
     else
         return RL_ERR_ARG;
     return rl_launch_status();
@@ -1455,5 +1505,74 @@ extern "C" int rl_read_buffer(const void* src, size_t bytes, unsigned* sink, int
     if (bytes < 16 || blocks < 1 || (reinterpret_cast<uintptr_t>(src) & 15)) return RL_ERR_ARG;
     hipLaunchKernelGGL(read_kernel, dim3(blocks), dim3(256), 0, stream, (const uint4*)src,
                        bytes / 16, sink);
+    return rl_launch_status();
+}
+
+// --------------------------------------------------------------------------- //
+// An activation over a token's whole hidden vector z (in place or not):
+//   out = a N(z) + b N(z^2) + c N(z^3) + e,   N(y) = y / sqrt(mean(y^2) + eps),
+// powers element by element, (a, b, c, e) = coef[0..3].  One workgroup a row; the three sums of
+// squares and the result are float32, and a row's sums are formed in one order whatever the step.
+// --------------------------------------------------------------------------- //
+template <typename T>
+__global__ __launch_bounds__(256) void polynorm_kernel(const T* __restrict__ x, T* __restrict__ out, int cols,
+                                                       const float* __restrict__ coef, float eps) {
+    __shared__ float scratch[16];
+    const T* row = x + (size_t)blockIdx.x * cols;
+    T* dst = out + (size_t)blockIdx.x * cols;
+    float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+    for (int i = threadIdx.x; i < cols; i += blockDim.x) {
+        const float z = to_float(row[i]);
+        const float z2 = z * z;
+        s2 += z2;
+        s4 += z2 * z2;
+        s6 += z2 * z2 * z2;
+    }
+    s2 = block_sum(s2, scratch);
+    s4 = block_sum(s4, scratch);
+    s6 = block_sum(s6, scratch);
+    const float r1 = coef[0] * rsqrtf(s2 / (float)cols + eps);
+    const float r2 = coef[1] * rsqrtf(s4 / (float)cols + eps);
+    const float r3 = coef[2] * rsqrtf(s6 / (float)cols + eps);
+    const float e = coef[3];
+    for (int i = threadIdx.x; i < cols; i += blockDim.x) {
+        const float z = to_float(row[i]);
+        dst[i] = from_float<T>(z * r1 + (z * z) * r2 + (z * z * z) * r3 + e);
+    }
+}
+
+extern "C" int rl_polynorm(const void* x, void* out, int tokens, int cols, const float* coef, float eps,
+                           int act_type, hipStream_t stream) {
+    if (tokens <= 0) return RL_OK;
+    if (cols < 1 || !coef) return RL_ERR_ARG;
+    if (act_type == RL_F32)
+        hipLaunchKernelGGL(polynorm_kernel<float>, dim3(tokens), dim3(256), 0, stream, (const float*)x, (float*)out,
+                           cols, coef, eps);
+    else if (act_type == RL_BF16)
+        hipLaunchKernelGGL(polynorm_kernel<bf16_t>, dim3(tokens), dim3(256), 0, stream, (const bf16_t*)x,
+                           (bf16_t*)out, cols, coef, eps);
+    else
+        return RL_ERR_ARG;
+    return rl_launch_status();
+}
+
+// --------------------------------------------------------------------------- //
+// Finished logits in place (float32): v <- v * scale, then, with cap > 0, v <- cap * tanh(v / cap)
+// --------------------------------------------------------------------------- //
+__global__ void scale_cap_kernel(float* __restrict__ v, size_t total, float scale, float cap) {
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (; idx < total; idx += step) {
+        const float y = v[idx] * scale;
+        v[idx] = cap > 0.f ? cap * tanhf(y / cap) : y;
+    }
+}
+
+extern "C" int rl_scale_cap(float* v, size_t total, float scale, float cap, hipStream_t stream) {
+    if (total == 0) return RL_OK;
+    if (cap < 0.f) return RL_ERR_ARG;
+    size_t blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(scale_cap_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, v, total, scale, cap);
     return rl_launch_status();
 }

@@ -26,6 +26,7 @@ import numpy as np
 
 from ..config.engine_config import EngineConfig
 from ..config.model_config import read_config_json
+from ..config.registry import config_from_dict
 from .step import ModelRunner, StepEntry
 
 REPLAY_PAGE_SIZE = 16
@@ -38,7 +39,9 @@ def build_replay_runner(model_dir: str | Path, dtype: str, max_tokens: int) -> M
     body = read_config_json(model_dir)
     page = REPLAY_PAGE_SIZE
     pages = -(-int(max_tokens) // page)
-    limit = int(body.get("max_position_embeddings", max_tokens))
+    # the longest sequence the architecture is defined for, as its model description says it
+    entry, config = config_from_dict(body)
+    limit = int(entry.build_spec(config).max_position or max_tokens)
     engine = EngineConfig(
         dtype=dtype,
         max_seq_len=max(2, min(limit, pages * page)),

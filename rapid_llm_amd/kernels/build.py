@@ -12,6 +12,8 @@ Two kinds of library exist:
 * ``attn_d<D>``: the matrix-core attention kernels, compiled for one head size ``D``.
   A model compiles only the head sizes it has.
 * ``mlstm``: the matrix-memory recurrence, compiled when a model has such a mixer.
+* ``recurrent``: the token-shift time mixing and the state-space mixer (scans, short convolution,
+  grouped norm), compiled when a model has such a mixer.
 * ``attn_tile_d<D>_v<DV>``: the tile attention for key heads of ``D`` and value heads of ``DV``
   channels, compiled when a model has a mixer that needs it.
 
@@ -47,6 +49,7 @@ CORE_SOURCES = (
 )
 ATTENTION_SOURCES = ("attention_mfma.hip", "attention_f32.hip")
 MLSTM_SOURCES = ("mlstm.hip",)
+RECURRENT_SOURCES = ("recurrent.hip",)
 ATTENTION_TILE_SOURCES = ("attention_tile.hip",)
 HEADERS = ("common.h", "static_entry.h")
 
@@ -226,6 +229,10 @@ def mlstm_library(force: bool = False) -> Path:
     return compile_library("mlstm", MLSTM_SOURCES, force=force)
 
 
+def recurrent_library(force: bool = False) -> Path:
+    return compile_library("recurrent", RECURRENT_SOURCES, force=force)
+
+
 def attention_tile_library(head_dim: int, value_dim: int, force: bool = False) -> Path:
     # beyond 320 / 256 channels a lane's operands no longer fit its registers: the compiler
     # parks some in scratch memory, which is slower and as exact
@@ -238,7 +245,7 @@ def attention_tile_library(head_dim: int, value_dim: int, force: bool = False) -
 
 def build_all(head_dims: tuple[int, ...] = DEFAULT_HEAD_DIMS, force: bool = True) -> list[Path]:
     """Compile every library (what ``__graft_entry__.build`` calls)."""
-    out = [core_library(force=force), mlstm_library(force=force)]
+    out = [core_library(force=force), mlstm_library(force=force), recurrent_library(force=force)]
     with ThreadPoolExecutor(8) as pool:
         out += list(pool.map(lambda pair: attention_tile_library(*pair, force=force), DEFAULT_TILE_HEAD_DIMS))
     if not all((CSRC / s).is_file() for s in ATTENTION_SOURCES):

@@ -107,6 +107,18 @@ def mlstm_lib() -> ctypes.CDLL:
     return _mlstm
 
 
+_recurrent: ctypes.CDLL | None = None
+
+
+def recurrent_lib() -> ctypes.CDLL:
+    global _recurrent
+    if _recurrent is None:
+        _recurrent = build.load(build.recurrent_library())
+        if _recurrent.rl_recurrent_max_head_dim() != WKV_MAX_HEAD_DIM or _recurrent.rl_conv_max_taps() != CONV_MAX_TAPS:
+            raise KernelError("the recurrence library's limits are not the launch rules'")
+    return _recurrent
+
+
 def _stream() -> ctypes.c_void_p:
     # the raw handle of the current stream of the current device, without the stream object
     # that ``torch.cuda.current_stream()`` builds (2.8 against 0.2 us a call, on every launch)
@@ -151,11 +163,13 @@ def _ok(code: int, what: str) -> None:
 
 def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, fed: Optional[torch.Tensor] = None,
           scale: float = 1.0, positions: Optional[torch.Tensor] = None,
-          inv_freq: Optional[torch.Tensor] = None) -> None:
+          inv_freq: Optional[torch.Tensor] = None, pos_table: Optional[torch.Tensor] = None) -> None:
     """``out[t] = table[ids[t]] * scale``; an id ``-(r + 1)`` takes ``fed[r]``, the token a
     sampling kernel chose in row ``r`` of the previous step.  With ``inv_freq`` (float32, one
     frequency per pair of channels) the sinusoidal vector of ``positions[t]`` is added: channel
-    ``2i`` gets the sine, ``2i + 1`` the cosine of the float32 product ``positions[t] * inv_freq[i]``."""
+    ``2i`` gets the sine, ``2i + 1`` the cosine of the float32 product ``positions[t] * inv_freq[i]``.
+    With ``pos_table`` (rows of the table's type) row ``positions[t]`` is added, unscaled; the
+    caller checks that every position has a row."""
     tokens = ids.numel()
     vocab, hidden = table.shape
     _need(ids, "ids", torch.int32)
@@ -168,11 +182,17 @@ def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, fed: Option
         if positions is None:
             raise KernelError("a sinusoidal position vector needs the tokens' positions")
         _need(positions, "positions", torch.int32, (tokens,))
+    if pos_table is not None:
+        _need(pos_table, "position table", table.dtype, (None, hidden))
+        if positions is None:
+            raise KernelError("learned position vectors need the tokens' positions")
+        _need(positions, "positions", torch.int32, (tokens,))
+    with_positions = inv_freq is not None or pos_table is not None
     _ok(
         core().rl_embed(
             _p(ids), _p(fed), 0 if fed is None else fed.numel(), _p(table), _tag(table.dtype), _p(out),
-            tokens, hidden, vocab, ctypes.c_float(scale), _p(positions if inv_freq is not None else None),
-            _p(inv_freq), _stream(),
+            tokens, hidden, vocab, ctypes.c_float(scale), _p(positions if with_positions else None),
+            _p(inv_freq), _p(pos_table), _stream(),
         ),
         "rl_embed",
     )
@@ -257,7 +277,7 @@ def pair_rows(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor) -> None:
     _ok(core().rl_pair_rows(_p(a), _p(b), _p(out), tokens, hidden, _tag(out.dtype), _stream()), "rl_pair_rows")
 
 
-UNARY_ACTIVATIONS = {"gelu_tanh": 0, "relu_squared": 1}
+UNARY_ACTIVATIONS = {"gelu_tanh": 0, "relu_squared": 1, "tanh": 2}
 
 
 def unary_act(x: torch.Tensor, out: torch.Tensor, kind: str, route: Optional[torch.Tensor] = None,
@@ -297,12 +317,20 @@ def route(logits: torch.Tensor, top: int, scale: float) -> None:
     _ok(core().rl_route(_p(logits), tokens, experts, top, ctypes.c_float(scale), _stream()), "rl_route")
 
 
-def router(x: torch.Tensor, w: torch.Tensor, top: int, scale: float, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+ROUTER_SCORES = {"softmax": 0, "sigmoid": 1}
+
+
+def router(x: torch.Tensor, w: torch.Tensor, top: int, scale: float, bias: Optional[torch.Tensor] = None,
+           scores: str = "softmax") -> torch.Tensor:
     """The experts' weights ``[tokens, experts]`` (float32) of rows ``x`` under the float32 router
     matrix ``w [experts, k]``: the product in float32 (plus ``bias``, one number an expert),
     softmax over all experts, the ``top`` largest scores over their sum (+ 1e-20) times ``scale``
-    (which is the softmax over the chosen logits alone), 0 elsewhere.  One kernel; a token's
-    result does not depend on the rest of the step."""
+    (which is the softmax over the chosen logits alone), 0 elsewhere.  With ``scores="sigmoid"`` an
+    expert's score is the sigmoid of its logit and a chosen expert's weight is its score times
+    ``scale``, not divided by anything.  One kernel; a token's result does not depend on the rest
+    of the step."""
+    if scores not in ROUTER_SCORES:
+        raise KernelError(f"router scores are one of {sorted(ROUTER_SCORES)}, not {scores!r}")
     tokens, k = x.shape
     experts = w.shape[0]
     _need(x, "x")
@@ -313,7 +341,7 @@ def router(x: torch.Tensor, w: torch.Tensor, top: int, scale: float, bias: Optio
         _need(bias, "router bias", torch.float32, (experts,))
     out = torch.empty((tokens, experts), dtype=torch.float32, device=x.device)
     _ok(core().rl_router(_p(x), _p(w), _p(out), tokens, k, experts, top, ctypes.c_float(scale), _p(bias),
-                         _tag(x.dtype), _stream()),
+                         ROUTER_SCORES[scores], _tag(x.dtype), _stream()),
         "rl_router")
     return out
 
@@ -322,12 +350,15 @@ GLU_ALPHA = 1.702  # the sigmoid's slope in the clamped gated activation
 
 
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor, limit: float = 0.0, alpha: float = GLU_ALPHA,
-           route: Optional[torch.Tensor] = None, expert_ff: int = 0) -> None:
+           route: Optional[torch.Tensor] = None, expert_ff: int = 0, route_input: bool = False) -> None:
     """The gated activation of a packed ``[gate | up]`` row.  ``limit`` 0: ``silu(g) * u``.
     ``limit > 0``: ``g' * sigmoid(alpha g') * (u' + 1)`` with ``g' = min(g, limit)`` and
     ``u' = clamp(u, -limit, limit)``.  With ``route`` (float32 ``[tokens, experts]``) the first
     ``experts * expert_ff`` hidden units are those of the experts side by side and expert ``e``'s
-    are multiplied by ``route[t, e]``."""
+    are multiplied by ``route[t, e]``; with ``route_input`` its gate and up values are, before the
+    activation (the expert read a scaled input)."""
+    if route_input and route is None:
+        raise KernelError("scaling the experts' inputs needs their weights")
     tokens, two_i = gate_up.shape
     if limit < 0:
         raise KernelError(f"the gated activation's limit must not be negative, got {limit}")
@@ -344,10 +375,33 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor, limit: float = 0.0, alpha: 
     _ok(
         core().rl_swiglu(
             _p(gate_up), _p(out), tokens, two_i // 2, _tag(out.dtype), ctypes.c_float(limit),
-            ctypes.c_float(alpha), _p(route), experts, int(expert_ff), _stream(),
+            ctypes.c_float(alpha), _p(route), experts, int(expert_ff), int(bool(route_input)), _stream(),
         ),
         "rl_swiglu",
     )
+
+
+def polynorm(x: torch.Tensor, out: torch.Tensor, coefficients: torch.Tensor, eps: float) -> None:
+    """``out = a N(x) + b N(x^2) + c N(x^3) + e`` row by row, with element-wise powers, ``N``
+    dividing a row by its root mean square (``eps`` inside the root) and ``coefficients`` =
+    ``(a, b, c, e)`` float32; sums and statistics float32.  ``out`` may be ``x``."""
+    tokens, cols = x.shape
+    _need(x, "x")
+    _need(out, "out", x.dtype, (tokens, cols))
+    _need(coefficients, "coefficients", torch.float32, (4,))
+    _ok(core().rl_polynorm(_p(x), _p(out), tokens, cols, _p(coefficients), ctypes.c_float(eps), _tag(x.dtype),
+                           _stream()),
+        "rl_polynorm")
+
+
+def scale_cap(values: torch.Tensor, scale: float, cap: float) -> None:
+    """In place on a float32 tensor: ``v * scale`` and then, with ``cap`` > 0, ``cap * tanh(v / cap)``."""
+    _need(values, "values", torch.float32)
+    if cap < 0:
+        raise KernelError(f"a cap must not be negative, got {cap}")
+    _ok(core().rl_scale_cap(_p(values), ctypes.c_size_t(values.numel()), ctypes.c_float(scale),
+                            ctypes.c_float(cap), _stream()),
+        "rl_scale_cap")
 
 
 def cast(src: torch.Tensor, dst: torch.Tensor) -> None:
@@ -516,12 +570,18 @@ def attention_generic(
     keep_first: int = 0,
     sink: bool = False,
     sink_values: Optional[torch.Tensor] = None,
+    score_cap: float = 0.0,
+    slopes: Optional[torch.Tensor] = None,
 ) -> None:
     tokens = q.shape[0]
     pages = k_cache.shape[0]
     dv = d if value_dim is None else int(value_dim)
     if sink_values is not None:
         _need(sink_values, "sink values", torch.float32, (nq,))
+    if slopes is not None:
+        _need(slopes, "distance slopes", torch.float32, (nq,))
+    if score_cap < 0:
+        raise KernelError(f"the cap of the scores must not be negative, got {score_cap}")
     _need(q, "q", None, (tokens, nq * d))
     _need(out, "out", q.dtype, (tokens, nq * dv))
     _need(k_cache, "k_cache", q.dtype, (pages, nkv, page_size, d))
@@ -539,7 +599,7 @@ def attention_generic(
             _p(q), _p(k_cache), _p(v_cache), _p(out), _p(positions), _p(token_slot),
             _p(block_table), block_table.stride(0), page_size, tokens, nq, nkv, d, window,
             ctypes.c_float(scale), dv, int(keep_first), int(bool(sink) or sink_values is not None),
-            _p(sink_values), _tag(q.dtype), _stream(),
+            _p(sink_values), ctypes.c_float(score_cap), _p(slopes), _tag(q.dtype), _stream(),
         ),
         "rl_attention_generic",
     )
@@ -1444,16 +1504,24 @@ def attention_tile(
     sink: bool,
     scale: float,
     sink_values: Optional[torch.Tensor] = None,
+    score_cap: float = 0.0,
+    slopes: Optional[torch.Tensor] = None,
 ) -> None:
     """Attention of every token of the step, in tiles of 16 rows on the matrix cores, for value
     heads of a size of their own, a window that keeps a request's first ``keep_first`` positions
     visible, and (``sink``) a softmax with 1 added to its denominator, or with ``sink_values``
-    (float32, one number a query head) ``exp`` of the head's number.  float32 (bit for bit the
-    same however the step was cut) or bfloat16."""
+    (float32, one number a query head) ``exp`` of the head's number.  ``score_cap`` c > 0 turns a
+    scaled score s into ``c * tanh(s / c)``; ``slopes`` (float32, one number a query head) then take
+    ``slope * (distance between query and key)`` off it.  float32 (bit for bit the same however
+    the step was cut) or bfloat16."""
     tokens = q.shape[0]
     if sink_values is not None:
         _need(sink_values, "sink values", torch.float32, (nq,))
         sink = True
+    if slopes is not None:
+        _need(slopes, "distance slopes", torch.float32, (nq,))
+    if score_cap < 0:
+        raise KernelError(f"the cap of the scores must not be negative, got {score_cap}")
     pages = k_cache.shape[0]
     _need(q, "q", None, (tokens, nq * d))
     _need(out, "out", q.dtype, (tokens, nq * dv))
@@ -1500,7 +1568,7 @@ def attention_tile(
             _p(q), _p(k_cache), _p(v_cache), _p(out), _p(tiles), num_tiles, _p(ctx.positions),
             _p(ctx.token_slot), _p(block_table), block_table.stride(0), page_size, nq, nkv, window,
             int(keep_first), int(bool(sink)), ctypes.c_float(scale), nsplit, _p(part), tokens, tile_rows,
-            _tag(q.dtype), _p(sink_values), _stream(),
+            _tag(q.dtype), _p(sink_values), ctypes.c_float(score_cap), _p(slopes), _stream(),
         ),
         "rl_attn_tile",
     )
@@ -1537,6 +1605,8 @@ def paged_attention(
     keep_first: int = 0,
     sink: bool = False,
     sink_values: Optional[torch.Tensor] = None,
+    score_cap: float = 0.0,
+    slopes: Optional[torch.Tensor] = None,
 ) -> None:
     """Attention of every token of the step over its request's cached keys.
 
@@ -1551,23 +1621,25 @@ def paged_attention(
     ``value_dim`` (the size of a value head, where it is not ``d``), ``keep_first`` (with a window:
     the request's first positions stay visible behind it) and ``sink`` (1 added to the softmax's
     denominator: a key of score 0 without a value; with ``sink_values`` its score is a number of
-    the query head, not scaled) send the step to the kernels that take them:
+    the query head, not scaled), ``score_cap`` (a scaled score s becomes ``cap * tanh(s / cap)``) and
+    ``slopes`` (one number a query head, times the distance between query and key, taken off the
+    score) send the step to the kernels that take them:
     tiles of 16 rows on the matrix cores for head sizes in steps of 16, the FMA kernel otherwise."""
     if prepare is not None and not attention_prepares_queries(q.dtype, d, 0 if prepare[1] is None else prepare[1].shape[1]):
         raise KernelError("the attention kernels do not finish the queries of this head size, type or rotation")
     dv = d if value_dim is None else int(value_dim)
     keep_first = int(keep_first) if window > 0 else 0  # without a window every key is seen anyway
-    if dv != d or keep_first or sink or sink_values is not None:
+    if dv != d or keep_first or sink or sink_values is not None or score_cap or slopes is not None:
         # value heads of their own size, kept first positions, one more term in the denominator
         if prepare is not None:
             raise KernelError("queries are finished before an attention with these options")
         if d % 16 == 0 and dv % 16 == 0 and page_size % 4 == 0:
             attention_tile(q, k_cache, v_cache, out, ctx, block_table, page_size, nq, nkv, d, dv,
-                           window, keep_first, sink, scale, sink_values)
+                           window, keep_first, sink, scale, sink_values, score_cap, slopes)
         else:
             attention_generic(
                 q, k_cache, v_cache, out, ctx.positions, ctx.token_slot, block_table, page_size,
-                nq, nkv, d, window, scale, ctx.max_position, dv, keep_first, sink, sink_values,
+                nq, nkv, d, window, scale, ctx.max_position, dv, keep_first, sink, sink_values, score_cap, slopes,
             )
         return
     if q.dtype == torch.float32 and d % 16 == 0:
@@ -1932,4 +2004,151 @@ def mlstm(
             ctypes.c_float(eps), _tag(packed.dtype), _stream(),
         ),
         "rl_mlstm_finish",
+    )
+
+
+# --------------------------------------------------------------------------- #
+# token-shift time mixing and the state-space mixer
+# --------------------------------------------------------------------------- #
+WKV_MAX_HEAD_DIM = 256  # a thread keeps one column of a head's state in registers
+SSM_MAX_STATE = 256
+SSM_MAX_HEAD_DIM = 256
+CONV_MAX_TAPS = 8
+
+
+def _step_requests(ctx, tokens: int, slots: int) -> None:
+    """The per-request tables every recurrent kernel walks, checked against the rows and the state."""
+    _need(ctx.cu_seqlens, "cu_seqlens", torch.int32, (ctx.num_seqs + 1,))
+    _need(ctx.seq_slots, "seq_slots", torch.int32, (ctx.num_seqs,))
+    if ctx.h_seq_slots and max(ctx.h_seq_slots) >= slots:
+        raise KernelError(f"slot {max(ctx.h_seq_slots)} is outside a state of {slots} slots")
+    if sum(ctx.h_seq_lens) != tokens or (ctx.h_seq_lens and min(ctx.h_seq_lens) < 1):
+        raise KernelError(f"the step's requests bring {list(ctx.h_seq_lens)} tokens, the rows are {tokens}")
+
+
+def token_shift(x: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, mixes: torch.Tensor, mix_last: torch.Tensor,
+                ctx) -> None:
+    """The five mixes of a token-shift mixer: with ``h'`` the row before a token's (the request's
+    ``state`` row, float32 ``[slots, width]``, before its first token of the step), branch ``b``
+    reads ``h + (h' - h) * mu[b]`` (``mu`` float32 ``[5 * width]``).  Branches 0 to 3 go to
+    ``mixes [4, tokens, width]`` in the type of ``x``, branch 4 to ``mix_last [tokens, width]`` in
+    float32.  Afterwards every request's state row holds its last row of the step."""
+    tokens, width = x.shape
+    _need(x, "x")
+    _need(mu, "mix coefficients", torch.float32, (5 * width,))
+    _need(state, "shift state", torch.float32, (None, width))
+    _need(mixes, "mixes", x.dtype, (4, tokens, width))
+    _need(mix_last, "float32 mix", torch.float32, (tokens, width))
+    _step_requests(ctx, tokens, state.shape[0])
+    _ok(
+        recurrent_lib().rl_token_shift(_p(x), _p(mu), _p(state), _p(mixes), _p(mix_last), _p(ctx.cu_seqlens),
+                                       _p(ctx.seq_slots), ctx.num_seqs, tokens, width, _tag(x.dtype), _stream()),
+        "rl_token_shift",
+    )
+
+
+def wkv(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, decay_pre: torch.Tensor,
+        decay_bias: torch.Tensor, bonus: torch.Tensor, norm_weight: torch.Tensor, out: torch.Tensor, ctx,
+        S: torch.Tensor, heads: int, d: int, eps: float) -> None:
+    """The time-mixing recurrence between its projections and its output projection.  ``r, k, v,
+    g [T, heads * d]``; ``decay_pre`` float32: the decay of a key channel is ``exp(-exp(decay_pre +
+    decay_bias))``; ``bonus [heads, d]`` weighs the current token's own key.  Per head, with the
+    state ``S [slots, heads, d, d]`` (float32, key channel first) read at the rows
+    ``ctx.seq_slots`` and left as it is after each request's last token::
+
+        o = (S + diag(bonus) k v^T)^T r        S <- diag(decay) S + k v^T
+
+    ``out``: every head's ``o`` divided by its root mean square (``eps`` inside the root), times
+    ``norm_weight``, times ``silu(g)``."""
+    tokens, inner = r.shape
+    if inner != heads * d or not 1 <= d <= WKV_MAX_HEAD_DIM:
+        raise KernelError(f"rows of {inner} are not {heads} heads of {d} (at most {WKV_MAX_HEAD_DIM}) channels")
+    for t, name in ((r, "r"), (k, "k"), (v, "v"), (g, "g"), (out, "out")):
+        _need(t, name, r.dtype, (tokens, inner))
+    _need(decay_pre, "decay pre-activations", torch.float32, (tokens, inner))
+    _need(decay_bias, "decay bias", torch.float32, (inner,))
+    _need(bonus, "bonus", torch.float32, (heads, d))
+    _need(norm_weight, "head norm weight", torch.float32, (inner,))
+    _need(S, "state", torch.float32, (None, heads, d, d))
+    _step_requests(ctx, tokens, S.shape[0])
+    _ok(
+        recurrent_lib().rl_wkv_scan(_p(r), _p(k), _p(v), _p(g), _p(decay_pre), _p(decay_bias), _p(bonus),
+                                    _p(norm_weight), _p(out), _p(ctx.cu_seqlens), _p(ctx.seq_slots), _p(S),
+                                    ctx.num_seqs, heads, d, ctypes.c_float(eps), _tag(r.dtype), _stream()),
+        "rl_wkv_scan",
+    )
+
+
+def causal_conv(packed: torch.Tensor, col0: int, weight: torch.Tensor, bias: torch.Tensor, state: torch.Tensor,
+                out: torch.Tensor, ctx) -> None:
+    """A causal convolution per channel over the columns ``col0 ..`` of ``packed``, with bias and
+    silu: ``weight [channels, taps]`` float32, whose last column meets the current token.  Inputs
+    before a request's first token of the step are its ``state`` rows (float32 ``[slots, taps - 1,
+    channels]``, oldest first; one row that is never read for a single tap), which afterwards hold
+    the last ``taps - 1`` inputs the request has seen.  ``out [tokens, channels]`` float32."""
+    tokens, width = packed.shape
+    channels, taps = weight.shape
+    _need(packed, "packed rows")
+    _need(weight, "convolution taps", torch.float32)
+    _need(bias, "convolution bias", torch.float32, (channels,))
+    _need(state, "convolution state", torch.float32, (None, max(taps - 1, 1), channels))
+    _need(out, "out", torch.float32, (tokens, channels))
+    if not 1 <= taps <= CONV_MAX_TAPS or col0 < 0 or col0 + channels > width:
+        raise KernelError(f"{taps} taps over columns {col0}..{col0 + channels} of rows of {width}")
+    _step_requests(ctx, tokens, state.shape[0])
+    _ok(
+        recurrent_lib().rl_causal_conv(_p(packed), width, int(col0), _p(weight), _p(bias), _p(state), _p(out),
+                                       _p(ctx.cu_seqlens), _p(ctx.seq_slots), ctx.num_seqs, tokens, channels, taps,
+                                       _tag(packed.dtype), _stream()),
+        "rl_causal_conv",
+    )
+
+
+def state_space_scan(mixed: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, decay_log: torch.Tensor,
+                     skip: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, ctx, S: torch.Tensor,
+                     heads: int, p: int, n: int, groups: int) -> None:
+    """The state-space recurrence.  ``mixed [T, heads * p + 2 * groups * n]`` float32: ``x``, ``B``
+    and ``C`` behind their convolution; ``dt_raw [T, heads]`` float32.  Per head (which reads group
+    ``head // (heads / groups)``), with ``dt = softplus(dt_raw + dt_bias)`` and the state ``S [slots,
+    heads, n, p]`` (float32) read at the rows ``ctx.seq_slots`` and left after each request's
+    last token::
+
+        S <- exp(-exp(decay_log) dt) S + dt B x^T        y = S^T C + skip x
+
+    ``out [T, heads * p]`` float32: ``y * silu(z)``, ``z`` the first ``heads * p`` columns of ``packed``."""
+    tokens = mixed.shape[0]
+    inner = heads * p
+    if groups < 1 or heads % groups or not 1 <= n <= SSM_MAX_STATE or not 1 <= p <= SSM_MAX_HEAD_DIM:
+        raise KernelError(f"{heads} heads of {p} channels in {groups} groups with states of {n}")
+    _need(mixed, "convolved rows", torch.float32, (tokens, inner + 2 * groups * n))
+    _need(dt_raw, "step sizes", torch.float32, (tokens, heads))
+    for t, name in ((dt_bias, "step bias"), (decay_log, "decay"), (skip, "skip")):
+        _need(t, name, torch.float32, (heads,))
+    _need(packed, "packed rows", None, (tokens, None))
+    if packed.shape[1] < inner:
+        raise KernelError(f"packed rows of {packed.shape[1]} hold no gate of {inner} channels")
+    _need(out, "out", torch.float32, (tokens, inner))
+    _need(S, "state", torch.float32, (None, heads, n, p))
+    _step_requests(ctx, tokens, S.shape[0])
+    _ok(
+        recurrent_lib().rl_ssm_scan(_p(mixed), _p(dt_raw), _p(dt_bias), _p(decay_log), _p(skip), _p(packed),
+                                    packed.shape[1], _p(out), _p(ctx.cu_seqlens), _p(ctx.seq_slots), _p(S),
+                                    ctx.num_seqs, heads, p, n, groups, _tag(packed.dtype), _stream()),
+        "rl_ssm_scan",
+    )
+
+
+def group_rmsnorm(y: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, parts: int, eps: float) -> None:
+    """Every row of ``y`` (float32) in ``parts`` equal parts, each divided by its own root mean
+    square (``eps`` inside the root), times ``weight``; ``out`` in either type."""
+    tokens, width = y.shape
+    _need(y, "y", torch.float32)
+    _need(weight, "norm weight", torch.float32, (width,))
+    _need(out, "out", None, (tokens, width))
+    if parts < 1 or width % parts:
+        raise KernelError(f"rows of {width} do not divide into {parts} parts")
+    _ok(
+        recurrent_lib().rl_group_rmsnorm(_p(y), _p(weight), _p(out), tokens, width, parts, ctypes.c_float(eps),
+                                         _tag(out.dtype), _stream()),
+        "rl_group_rmsnorm",
     )

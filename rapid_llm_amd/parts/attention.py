@@ -70,6 +70,10 @@ class GQAAttention(Mixer):
         value_dim: int | None = None,
         keep_first: int = 0,
         sink: bool = False,
+        sink_name: str | None = None,
+        qk_norm_weights: bool = True,
+        score_cap: float = 0.0,
+        distance_slope_exponent: float | None = None,
     ) -> None:
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are not divisible by {num_kv_heads} kv heads")
@@ -87,7 +91,15 @@ class GQAAttention(Mixer):
         if keep_first < 0:
             raise ValueError(f"a window keeps a number of first positions, not {keep_first}")
         self.keep_first = int(keep_first) if window else 0  # without a window every key is seen
-        self.sink = bool(sink)
+        self.sink = bool(sink) or sink_name is not None
+        self.sink_name = sink_name
+        self.sink_values = None
+        self.qk_norm_weights = bool(qk_norm_weights)
+        if score_cap < 0:
+            raise ValueError(f"the cap of the scores must not be negative, got {score_cap}")
+        self.score_cap = float(score_cap)
+        self.slope_exponent = None if distance_slope_exponent is None else float(distance_slope_exponent)
+        self.slopes = None
         self.prefix = checkpoint_prefix
         self.qk_norm_eps = qk_norm_eps
         self.window = int(window)
@@ -116,7 +128,8 @@ class GQAAttention(Mixer):
         self.gate_rows = num_heads if head_gate_name else 0
         self.gate_pad = -(self.qkv_rows + self.gate_rows) % 8 if self.gate_rows else 0
         # the options that only the tile kernels (or the kernel for any size) take
-        self.extended = self.dv != head_dim or self.keep_first > 0 or self.sink
+        self.extended = (self.dv != head_dim or self.keep_first > 0 or self.sink or self.score_cap > 0
+                         or self.slope_exponent is not None)
         self.plain_row = not self.values_are_keys and not self.gate_rows and not self.extended
         self.row_pad = -self.qkv_rows % 8 if (self.extended and not self.gate_rows) else 0
         self.qkv = Linear(hidden_size, self.qkv_rows + self.gate_rows + self.gate_pad + self.row_pad)
@@ -144,7 +157,9 @@ class GQAAttention(Mixer):
             ParamSpec(self.name + ".o", (self.hidden_size, self.nq * self.dv), "matrix",
                       (Source(p + n["o"], self.hidden_size),)),
         ]
-        if self.qk_norm_eps is not None:
+        if self.sink_name is not None:
+            specs.append(ParamSpec(self.name + ".sink", (self.nq,), "vector", (Source(p + self.sink_name, self.nq),)))
+        if self.qk_norm_eps is not None and self.qk_norm_weights:
             specs += [
                 ParamSpec(self.name + ".q_norm", (self.d,), "vector", (Source(p + n["qn"], self.d),), init="norm"),
                 ParamSpec(self.name + ".k_norm", (self.d,), "vector", (Source(p + n["kn"], self.d),), init="norm"),
@@ -178,9 +193,17 @@ class GQAAttention(Mixer):
         self.bias_in_kernel = None if self.plain_row else bias
         self.qkv.bind(params[self.name + ".qkv"], bias if self.plain_row else None)
         self.o.bind(params[self.name + ".o"], params[self.name + ".o_bias"] if self.o_bias else None)
-        if self.qk_norm_eps is not None:
+        if self.qk_norm_eps is not None and self.qk_norm_weights:
             self.q_norm_w = params[self.name + ".q_norm"]
             self.k_norm_w = params[self.name + ".k_norm"]
+        elif self.qk_norm_eps is not None:
+            # a norm without a learned weight: the kernels get a weight of ones
+            self.q_norm_w = self.k_norm_w = torch.ones(self.d, dtype=torch.float32, device=runtime.device)
+        if self.sink_name is not None:
+            self.sink_values = params[self.name + ".sink"]
+        if self.slope_exponent is not None:
+            h = torch.arange(1, self.nq + 1, dtype=torch.float64)
+            self.slopes = torch.exp2(-self.slope_exponent * h / self.nq).to(torch.float32).to(runtime.device)
         self.runtime = runtime
 
     # ---- cache -----------------------------------------------------------------
@@ -238,7 +261,8 @@ class GQAAttention(Mixer):
             qkv if in_kernel else q, cache.k, cache.v, out, ctx, table, cache.page_size,
             self.nq, self.nkv, self.d, self.window, self.scale,
             prepare=(self.q_norm_w, cos, sin, eps) if in_kernel else None,
-            value_dim=self.dv, keep_first=self.keep_first, sink=self.sink,
+            value_dim=self.dv, keep_first=self.keep_first, sink=self.sink, sink_values=self.sink_values,
+            score_cap=self.score_cap, slopes=self.slopes,
         )
         if self.gate_rows:
             ops.head_gate(out, qkv, self.qkv_rows, self.nq, self.d)

@@ -68,6 +68,10 @@ class ParamSpec:
     ``fallback`` names another parameter whose tensor is shared when the checkpoint has
     none of this one's sources (a tied output projection).
     ``init`` is the distribution the random-weights mode draws the sources from.
+
+    A ``shape`` of ``()`` is one number, which its single source feeds whole.  A size of ``-1``
+    in the shape of a parameter with one source is whatever the checkpoint's tensor has there (a
+    size that no configuration key gives); the random-weights mode cannot draw such a parameter.
     """
 
     name: str
@@ -80,6 +84,8 @@ class ParamSpec:
 
     def source_shape(self, rows: int) -> tuple[int, ...]:
         """Shape of a checkpoint tensor that feeds ``rows`` of this parameter's ``axis``."""
+        if not self.shape:
+            return ()
         return (*self.shape[: self.axis], rows, *self.shape[self.axis + 1 :])
 
 

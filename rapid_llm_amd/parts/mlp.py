@@ -79,7 +79,12 @@ class SwiGLU(FeedForward):
 
 class TwoLayer(FeedForward):
     """``down(act(up(x)))`` with a one-operand activation (``ops.UNARY_ACTIVATIONS``: the tanh form
-    of gelu, or the square of relu); no gate, no biases."""
+    of gelu, or the square of relu); no gate, no biases.
+
+    ``activation="polynorm"`` acts on a token's whole hidden vector ``z`` instead: ``a N(z) + b N(z^2)
+    + c N(z^3) + e`` with element-wise powers, ``N`` dividing a vector by its root mean square
+    (``activation_eps`` inside the root) and the four learned numbers ``a, b, c, e`` of the tensor
+    ``activation_name``; statistics and sums are float32."""
 
     replayable = True
 
@@ -92,9 +97,16 @@ class TwoLayer(FeedForward):
         name: str = "ff",
         up_name: str = "up",
         down_name: str = "down",
+        activation_name: str = "act",
+        activation_eps: float = 0.0,
     ) -> None:
-        if activation not in ops.UNARY_ACTIVATIONS:
-            raise ValueError(f"activation {activation!r} is not one of {sorted(ops.UNARY_ACTIVATIONS)}")
+        self.polynorm = activation == "polynorm"
+        if not self.polynorm and activation not in ops.UNARY_ACTIVATIONS:
+            raise ValueError(f"activation {activation!r} is not 'polynorm' or one of {sorted(ops.UNARY_ACTIVATIONS)}")
+        if self.polynorm and not activation_eps > 0:
+            raise ValueError(f"the normalised powers need a positive epsilon, got {activation_eps}")
+        self.activation_name, self.activation_eps = activation_name, float(activation_eps)
+        self.coefficients = None
         self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
         self.prefix, self.activation, self.name = checkpoint_prefix, activation, name
         self.names = (up_name, down_name)
@@ -104,18 +116,27 @@ class TwoLayer(FeedForward):
     def param_specs(self) -> list[ParamSpec]:
         h, i = self.hidden_size, self.intermediate_size
         u, d = (self.prefix + n for n in self.names)
-        return [
+        specs = [
             ParamSpec(self.name + ".up", (i, h), "matrix", (Source(u, i),)),
             ParamSpec(self.name + ".down", (h, i), "matrix", (Source(d, h),)),
         ]
+        if self.polynorm:
+            specs.append(ParamSpec(self.name + ".act", (4,), "vector", (Source(self.prefix + self.activation_name, 4),),
+                                   init="norm"))
+        return specs
 
     def bind(self, params, runtime) -> None:
         self.up.bind(params[self.name + ".up"])
         self.down.bind(params[self.name + ".down"])
+        if self.polynorm:
+            self.coefficients = params[self.name + ".act"]
 
     def forward(self, x, ctx):
         hidden = self.up(x)
-        ops.unary_act(hidden, hidden, self.activation)
+        if self.polynorm:
+            ops.polynorm(hidden, hidden, self.coefficients, self.activation_eps)
+        else:
+            ops.unary_act(hidden, hidden, self.activation)
         return self.down.deferred(hidden, ctx)
 
 
@@ -124,8 +145,13 @@ class RoutedExperts(FeedForward):
     scores highest, weighted by their scores over the chosen ones' sum (which is the softmax over
     the chosen logits alone), times ``route_scale``; a shared expert (``shared_size`` > 0) runs for
     every token and is added.  ``gated``: the experts are gated ones, ``down(silu(gate(x)) * up(x))``;
-    their gate and up projections form one packed matrix, all gates first.  ``router_bias_name``:
-    the router's logits get a bias, one number an expert.
+    their gate and up projections form one packed matrix, all gates first; with ``limit`` > 0 their
+    activation is the clamped one, ``g' * sigmoid(alpha g') * (u' + 1)``.  ``router_bias_name``:
+    the router's logits get a bias, one number an expert.  ``scores="sigmoid"``: an expert's score
+    is the sigmoid of its logit, and the chosen experts' weights are their scores as they are
+    (times ``route_scale``), not divided by their sum.  ``weights_scale="input"`` (gated experts): the
+    weight multiplies what the expert reads, not what it returns; its first products being linear,
+    the gate and up values are multiplied by it before they are clamped.
 
     The router's product and scores are float32 in every engine (its matrix is held in
     float32).  The experts' up projections are one packed matrix ``[experts * expert_size +
@@ -157,8 +183,20 @@ class RoutedExperts(FeedForward):
         gated: bool = False,
         gate_name: str = "gate",
         router_bias_name: str | None = None,
+        limit: float = 0.0,
+        alpha: float = ops.GLU_ALPHA,
+        scores: str = "softmax",
+        weights_scale: str = "output",
     ) -> None:
         self.gated = bool(gated)
+        if scores not in ops.ROUTER_SCORES:
+            raise ValueError(f"router scores are one of {sorted(ops.ROUTER_SCORES)}, not {scores!r}")
+        if weights_scale not in ("output", "input") or (weights_scale == "input" and not gated):
+            raise ValueError(f"an expert's weight scales its 'output', or the 'input' of a gated expert, not {weights_scale!r}")
+        if limit < 0 or (limit and not gated):
+            raise ValueError(f"a limit of {limit} needs gated experts and must not be negative")
+        self.limit, self.alpha, self.scores = float(limit), float(alpha), scores
+        self.scale_input = weights_scale == "input"
         if self.gated:
             if activation != "silu":
                 raise ValueError(f"gated experts use the silu gate, not {activation!r}")
@@ -212,11 +250,12 @@ class RoutedExperts(FeedForward):
 
     def forward(self, x, ctx):
         # float32 throughout
-        weights = ops.router(x, self.router.weight, self.top, self.route_scale, self.router_bias)
+        weights = ops.router(x, self.router.weight, self.top, self.route_scale, self.router_bias, self.scores)
         hidden = self.up(x)
         if self.gated:
             act = torch.empty((x.shape[0], self.inner), dtype=hidden.dtype, device=x.device)
-            ops.swiglu(hidden, act, route=weights, expert_ff=self.expert_size)
+            ops.swiglu(hidden, act, self.limit, self.alpha, route=weights, expert_ff=self.expert_size,
+                       route_input=self.scale_input)
             return self.down.deferred(act, ctx)
         ops.unary_act(hidden, hidden, self.activation, weights, self.expert_size)
         return self.down.deferred(hidden, ctx)

@@ -19,14 +19,20 @@ class RMSNorm(Norm):
     replayable = True
     fuses_products = True  # takes a DeferredProduct as delta, may return ScaledRows
 
-    def __init__(self, size: int, eps: float, checkpoint_name: str, name: str = "norm") -> None:
+    def __init__(self, size: int, eps: float, checkpoint_name: str, name: str = "norm",
+                 single_weight: bool = False) -> None:
         self.size = size
         self.eps = float(eps)
         self.checkpoint_name = checkpoint_name
         self.name = name
+        # one learned number for all coordinates instead of one a coordinate: the kernels get it
+        # laid out as a vector, so every fused form of the norm serves both
+        self.single_weight = bool(single_weight)
         self.weight: torch.Tensor | None = None
 
     def param_specs(self) -> list[ParamSpec]:
+        if self.single_weight:
+            return [ParamSpec(self.name + ".weight", (), "vector", (Source(self.checkpoint_name, 1),), init="norm")]
         return [
             ParamSpec(
                 self.name + ".weight",
@@ -39,6 +45,8 @@ class RMSNorm(Norm):
 
     def bind(self, params, runtime) -> None:
         self.weight = params[self.name + ".weight"]
+        if self.single_weight:
+            self.weight = self.weight.reshape(1).expand(self.size).contiguous()
         self.dtype = runtime.dtype
 
     def forward(self, residual, delta, ctx, rows=None, scaled_ok=False):

@@ -116,7 +116,7 @@ def load_params(
                 other.append(f"checkpoint tensor {src.name!r} is claimed by two parameters")
             by_source[src.name] = (spec, offset, src.rows)
             offset += src.rows
-        if spec.sources and offset != spec.shape[spec.axis]:
+        if spec.sources and spec.shape and offset != spec.shape[spec.axis] and spec.shape[spec.axis] != -1:
             other.append(
                 f"parameter {spec.name!r}: its sources cover {offset} rows of {spec.shape[spec.axis]}"
             )
@@ -137,6 +137,12 @@ def load_params(
         seen.add(name)
         spec, offset, rows = hit
         want = spec.source_shape(rows)
+        free = -1 in spec.shape  # sizes that the checkpoint's tensor gives (one source only)
+        if free and (len(spec.sources) != 1 or len(want) != tensor.dim()):
+            wrong.append(f"{name}: checkpoint has {tuple(tensor.shape)}, parameter {spec.name!r} expects {want}")
+            continue
+        if free:
+            want = tuple(have if w == -1 else w for w, have in zip(spec.shape, tensor.shape))
         if tuple(tensor.shape) != want:
             wrong.append(
                 f"{name}: checkpoint has {tuple(tensor.shape)}, parameter {spec.name!r} "
@@ -154,14 +160,17 @@ def load_params(
         dtype = storage_dtype(spec.role, tensor.dtype, engine_dtype)
         if dest is None:
             padded = any(not s.name for s in spec.sources)
-            dest = (torch.zeros if padded else torch.empty)(spec.shape, dtype=dtype, device=device)
+            dest = (torch.zeros if padded else torch.empty)(want if free else spec.shape, dtype=dtype, device=device)
             out[spec.name] = dest
         elif dest.dtype != dtype:
             # blocks of one fused matrix stored in different widths: keep the wider
             if dtype == torch.float32:
                 dest = dest.to(torch.float32)
                 out[spec.name] = dest
-        dest.narrow(spec.axis, offset, rows).copy_(tensor, non_blocking=False)
+        if free or not spec.shape:
+            dest.copy_(tensor, non_blocking=False)
+        else:
+            dest.narrow(spec.axis, offset, rows).copy_(tensor, non_blocking=False)
 
     missing: list[str] = []
     for spec in specs:

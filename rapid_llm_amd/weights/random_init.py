@@ -25,6 +25,8 @@ _STORE = {"bfloat16": torch.bfloat16, "float32": torch.float32}
 
 
 def _draw(shape, init: str, gen: torch.Generator, std: float, norm_std: float, device="cpu"):
+    if -1 in tuple(shape):
+        raise ValueError(f"a tensor of shape {tuple(shape)} takes a size from a checkpoint; random weights need it given")
     if init == "norm":
         t = torch.ones(shape, dtype=torch.float32, device=device)
         if norm_std:
