@@ -3,7 +3,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--dtype bfloat16]
                     [--shape NAME] [--batch B] [--prompt-len T] [--context C]
     python bench.py --workload qwen3-0.6b-256 | qwen3-32b-32
-    python bench.py --design fokulorn|sikevik|miborax [--design-size 2b,8b]
+    python bench.py --design fokulorn|sikevik|miborax|fomunex [--design-size 2b,8b]
 
 A "step" is one decode step of the whole batch through the engine's step function and the
 greedy sampling kernel, tokens fed back.  The default run has the layer sizes of
@@ -41,6 +41,13 @@ all heads share, half of the layers windowed, a quarter reading the rows another
 sub-layers of a layer behind layer norms of the same stream; mixtures of eight gated experts with a
 router bias), beside the Sikevik decoder, the engine's closest (a sink term, windows, routed
 experts), and Qwen3 of equal size.
+
+``--design fomunex`` does the same for the Fomunex decoder (layers in turn: capped windowed
+attention with a distance term and learned sinks, a token-shift time mixing, a state-space mixer
+behind a short convolution, attention again; dense feed-forwards with a polynomial activation in
+the even layers, mixtures of eight clamped gated experts behind a sigmoid router in the odd ones),
+beside the Fokulorn decoder, the engine's closest (recurrent layers with a state per request
+beside windowed attention), and Qwen3 of equal size.
 
 Metric definitions follow rapid_llm's docs/benchmark_models.md:141-149: decode tok/s is
 batch / mean step time; prefill tok/s is prompt tokens / prefill latency; both timed
@@ -652,12 +659,153 @@ def _time_miborax_kernels(z: dict, prompt_len: int, batch: int) -> dict:
     return out
 
 
+def fomunex_body(z: dict) -> dict:
+    """Layers in turn attention, time mixing, state-space, attention; the recurrent mixers with
+    heads of 64 channels (the time mixing as wide as the model, the state-space mixer twice as
+    wide with states of 128); a layer's feed-forward matrices hold what Qwen3's three do."""
+    w, ff = z["width"], z["ff"]
+    attention = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["head_dim"], "vdim": z["head_dim"],
+                 "scale": z["head_dim"] ** -0.5, "softcap": 50.0, "mask": {"size": z["window"]}}
+    mixing = {"heads": w // 64, "dim": 64, "rank": 64}
+    space = {"heads": 2 * w // 64, "vdim": 64, "state": 128, "groups": 8, "conv": 4, "norm_groups": 8}
+    dense = {"kind": "dense", "ff": ff * 3 // 2}
+    moe = {"kind": "moe", "expert": {"ff": ff // 8, "limit": 7.0}, "router": {"experts": 8, "top": 2}}
+    kinds = [("attention", attention), ("wkv", mixing), ("mamba2", space), ("attention", attention)]
+    layers = [{"type": kinds[i % 4][0], "mixer": kinds[i % 4][1], "mlp": dense if i % 2 == 0 else moe}
+              for i in range(z["layers"])]
+    return {"architecture": "Fomunex", "width": w, "vocab": z["vocab"], "max_positions": 4096, "norm": {"eps": 1e-6},
+            "logit_scale": 1.0, "logit_softcap": 30.0, "layers": layers}
+
+
+def _time_fomunex_kernels(z: dict, prompt_len: int, batch: int) -> dict:
+    """The design's own kernels alone, microseconds and share of the roofline each.  The two scans
+    over one prompt (float32 operations: per token and head four a state element for the time
+    mixing, whose output reads the state before and its update after, and four for the state-space
+    one) and over ``batch`` single tokens (bytes of state read and written); the mixes, the
+    convolution and the polynomial activation (bytes); attention with cap, distance term and
+    learned sinks over one prompt from its start (matrix rate over the keys every query sees) and
+    over ``batch`` single tokens behind ``prompt_len`` (bytes of keys and values)."""
+    import types
+
+    import torch
+
+    from rapid_llm_amd.kernels import ops
+
+    dev, width = "cuda", z["width"]
+    bf = torch.bfloat16
+    out: dict = {}
+
+    def step(lens):
+        cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32, device=dev)
+        return types.SimpleNamespace(num_seqs=len(lens), h_seq_lens=list(lens), h_seq_slots=list(range(len(lens))),
+                                     cu_seqlens=cu, seq_slots=torch.arange(len(lens), dtype=torch.int32, device=dev))
+
+    # ---- time mixing
+    h, d = width // 64, 64
+    inner = h * d
+    S = torch.zeros((batch + 1, h, d, d), device=dev)
+    shift = torch.zeros((batch + 1, width), device=dev)
+    for what, lens in (("prefill", [prompt_len]), ("decode", [1] * batch)):
+        tokens, ctx = sum(lens), step(lens)
+        r, k, v, g = ((torch.randn(tokens, inner, device=dev) * 0.5).to(bf) for _ in range(4))
+        pre = torch.randn(tokens, inner, device=dev)
+        bias, u, nw = torch.full((inner,), -2.5, device=dev), torch.zeros((h, d), device=dev), torch.ones(inner, device=dev)
+        o = torch.empty((tokens, inner), dtype=bf, device=dev)
+        sec = _time_calls(lambda: ops.wkv(r, k, v, g, pre, bias, u, nw, o, ctx, S, h, d, 1e-6), what == "decode")
+        out[f"time_mixing_scan_{what}_us"] = round(sec * 1e6, 1)
+        if what == "prefill":
+            out["time_mixing_scan_prefill_frac_fp32_matrix"] = round(
+                tokens * h * 4.0 * d * d / sec / (PEAK_TFLOPS["float32"] * 1e12), 4)
+        else:
+            out["time_mixing_scan_decode_frac_hbm"] = round(2.0 * batch * h * d * d * 4 / sec / 1e9 / HBM_GBPS, 4)
+        x = (torch.randn(tokens, width, device=dev)).to(bf)
+        mu = torch.rand(5 * width, device=dev)
+        mixes, last = torch.empty((4, tokens, width), dtype=bf, device=dev), torch.empty((tokens, width), device=dev)
+        sec = _time_calls(lambda: ops.token_shift(x, mu, shift, mixes, last, ctx), what == "decode")
+        out[f"token_shift_{what}_us"] = round(sec * 1e6, 1)
+        out[f"token_shift_{what}_frac_hbm"] = round(tokens * width * (2 + 4 * 2 + 4) / sec / 1e9 / HBM_GBPS, 4)
+    # ---- state-space mixer
+    hs, P, N, G, taps = 2 * width // 64, 64, 128, 8, 4
+    inner = hs * P
+    channels = inner + 2 * G * N
+    S2 = torch.zeros((batch + 1, hs, N, P), device=dev)
+    conv_state = torch.zeros((batch + 1, taps - 1, channels), device=dev)
+    conv_w, conv_b = torch.randn(channels, taps, device=dev) * 0.5, torch.zeros(channels, device=dev)
+    for what, lens in (("prefill", [prompt_len]), ("decode", [1] * batch)):
+        tokens, ctx = sum(lens), step(lens)
+        packed = (torch.randn(tokens, inner + channels, device=dev) * 0.5).to(bf)
+        mixed = torch.empty((tokens, channels), device=dev)
+        sec = _time_calls(lambda: ops.causal_conv(packed, inner, conv_w, conv_b, conv_state, mixed, ctx), what == "decode")
+        out[f"convolution_{what}_us"] = round(sec * 1e6, 1)
+        out[f"convolution_{what}_frac_hbm"] = round(tokens * channels * (2 + 4) / sec / 1e9 / HBM_GBPS, 4)
+        dt = torch.randn(tokens, hs, device=dev)
+        vec = torch.zeros(hs, device=dev)
+        y = torch.empty((tokens, inner), device=dev)
+        sec = _time_calls(lambda: ops.state_space_scan(mixed, dt, vec - 1.0, vec - 1.0, vec + 1.0, packed, y, ctx, S2,
+                                                       hs, P, N, G), what == "decode")
+        out[f"state_space_scan_{what}_us"] = round(sec * 1e6, 1)
+        if what == "prefill":
+            out["state_space_scan_prefill_frac_fp32_matrix"] = round(
+                tokens * hs * 4.0 * N * P / sec / (PEAK_TFLOPS["float32"] * 1e12), 4)
+        else:
+            out["state_space_scan_decode_frac_hbm"] = round(2.0 * batch * hs * N * P * 4 / sec / 1e9 / HBM_GBPS, 4)
+        o = torch.empty((tokens, inner), dtype=bf, device=dev)
+        sec = _time_calls(lambda: ops.group_rmsnorm(y, torch.ones(inner, device=dev), o, 8, 1e-6), what == "decode")
+        out[f"norm_in_parts_{what}_us"] = round(sec * 1e6, 1)
+        out[f"norm_in_parts_{what}_frac_hbm"] = round(tokens * inner * (4 + 2) / sec / 1e9 / HBM_GBPS, 4)
+    # ---- the polynomial activation over a prompt's hidden rows
+    ff = z["ff"] * 3 // 2
+    hidden = (torch.randn(prompt_len, ff, device=dev)).to(bf)
+    coef = torch.tensor([0.7, 0.2, 0.1, 0.0], device=dev)
+    sec = _time_calls(lambda: ops.polynorm(hidden, hidden, coef, 1e-6), False)
+    out["polynomial_activation_prefill_us"] = round(sec * 1e6, 1)
+    out["polynomial_activation_prefill_frac_hbm"] = round(prompt_len * ff * 4 / sec / 1e9 / HBM_GBPS, 4)
+    # ---- attention
+    nq, nkv, dh, window, page = z["heads"], z["kv_heads"], z["head_dim"], z["window"], 16
+    sink = torch.zeros(nq, device=dev)
+    slopes = torch.exp2(-8.0 * torch.arange(1, nq + 1, device=dev, dtype=torch.float32) / nq)
+
+    def attention(seqs, plain):
+        tokens = sum(n for _, n in seqs)
+        pages_per = [-(-(a + n) // page) for a, n in seqs]
+        table = torch.zeros((len(seqs), max(pages_per)), dtype=torch.int32)
+        at = 1
+        for i, n in enumerate(pages_per):
+            table[i, :n] = torch.arange(at, at + n, dtype=torch.int32)
+            at += n
+        kc = (torch.randn(at, nkv, page, dh, device=dev) * 0.3).to(bf)
+        vc = (torch.randn(at, nkv, dh, page, device=dev) * 0.3).to(bf)
+        q = (torch.randn(tokens, nq * dh, device=dev) * 0.3).to(bf)
+        o = torch.empty((tokens, nq * dh), dtype=bf, device=dev)
+        positions = torch.cat([torch.arange(a, a + n) for a, n in seqs]).to(torch.int32).to(dev)
+        slot = torch.cat([torch.full((n,), i) for i, (_, n) in enumerate(seqs)]).to(torch.int32).to(dev)
+        ctx = types.SimpleNamespace(positions=positions, token_slot=slot, token_ids=positions,
+                                    h_seq_starts=[a for a, _ in seqs], h_seq_lens=[n for _, n in seqs],
+                                    max_position=max(a + n for a, n in seqs) - 1, extra={}, static={})
+        table = table.to(dev)
+        more = dict(sink=True) if plain else dict(sink_values=sink, score_cap=50.0, slopes=slopes)
+        return _time_calls(lambda: ops.paged_attention(q, kc, vc, o, ctx, table, page, nq, nkv, dh, window,
+                                                       dh ** -0.5, **more), max(n for _, n in seqs) == 1)
+
+    seen = sum(min(p + 1, window) for p in range(prompt_len))
+    for label, plain in (("", False), ("_without_cap_and_distance", True)):
+        sec = attention([(0, prompt_len)], plain)
+        out[f"attention_prefill{label}_us"] = round(sec * 1e6, 1)
+        out[f"attention_prefill{label}_frac_bf16_matrix"] = round(4.0 * nq * dh * seen / sec / (PEAK_TFLOPS["bfloat16"] * 1e12), 4)
+        sec = attention([(prompt_len, 1)] * batch, plain)
+        out[f"attention_decode{label}_us"] = round(sec * 1e6, 1)
+        out[f"attention_decode{label}_frac_hbm"] = round(
+            batch * min(prompt_len + 1, window) * nkv * dh * 2 * 2 / sec / 1e9 / HBM_GBPS, 4)
+    return out
+
+
 # design -> (name, its configuration at a size, its kernels alone, the engine's closest other
 # architecture measured beside it and Qwen3)
 DESIGNS = {
     "fokulorn": ("Fokulorn", fokulorn_body, _time_kernels, None),
     "sikevik": ("Sikevik", sikevik_body, _time_sikevik_kernels, None),
     "miborax": ("Miborax", miborax_body, _time_miborax_kernels, ("sikevik", sikevik_body)),
+    "fomunex": ("Fomunex", fomunex_body, _time_fomunex_kernels, ("fokulorn", fokulorn_body)),
 }
 
 
@@ -715,7 +863,7 @@ def main() -> int:
     ap.add_argument("--peaks", action="store_true",
                     help="measure what the device reaches with library kernels (a large read, copy and square products) and exit")
     ap.add_argument("--design", default=None,
-                    help="measure another architecture of the engine beside Qwen3 at equal size (fokulorn, sikevik, miborax) and exit")
+                    help="measure another architecture of the engine beside Qwen3 at equal size (fokulorn, sikevik, miborax, fomunex) and exit")
     ap.add_argument("--design-size", default="2b,8b", help=f"sizes for --design: {', '.join(DESIGN_SIZES)}")
     args = ap.parse_args()
     if args.peaks:

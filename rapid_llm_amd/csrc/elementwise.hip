@@ -23,10 +23,11 @@ template <typename W>
 __global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict__ fed, int fed_rows,
                              const W* __restrict__ table, float* __restrict__ out, int hidden,
                              int vocab, float scale, const int* __restrict__ positions,
-                             const float* __restrict__ inv_freq, const W* __restrict__ pos_table) {
+                             const float* __restrict__ inv_freq, const W* __restrict__ pos_table, int pos_rows) {
     const int t = blockIdx.x;
     const int pos = (inv_freq || pos_table) ? positions[t] : 0;
-    const W* prow = pos_table ? pos_table + (size_t)pos * hidden : nullptr;
+    // positions are validated on the host; one beyond the table reads its last row rather than faulting
+    const W* prow = pos_table ? pos_table + (size_t)min(max(pos, 0), pos_rows - 1) * hidden : nullptr;
     int id = ids[t];
     if (id < 0 && fed && -id - 1 < fed_rows) id = fed[-id - 1];
     // ids are validated on the host; an id outside the table reads row 0 rather than faulting
@@ -73,18 +74,20 @@ __global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict_
 
 extern "C" int rl_embed(const int* ids, const int* fed, int fed_rows, const void* table,
                         int table_type, float* out, int tokens, int hidden, int vocab, float scale,
-                        const int* positions, const float* inv_freq, const void* pos_table, hipStream_t stream) {
+                        const int* positions, const float* inv_freq, const void* pos_table, int pos_rows,
+                        hipStream_t stream) {
     if (tokens <= 0) return RL_OK;
     if ((inv_freq || pos_table) && !positions) return RL_ERR_ARG;
+    if (pos_table && pos_rows < 1) return RL_ERR_ARG;
     dim3 grid(tokens), block(256);
     if (table_type == RL_F32)
         hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, ids, fed, fed_rows,
                            (const float*)table, out, hidden, vocab, scale, positions, inv_freq,
-                           (const float*)pos_table);
+                           (const float*)pos_table, pos_rows);
     else if (table_type == RL_BF16)
         hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, ids, fed, fed_rows,
                            (const bf16_t*)table, out, hidden, vocab, scale, positions, inv_freq,
-                           (const bf16_t*)pos_table);
+                           (const bf16_t*)pos_table, pos_rows);
     else
         return RL_ERR_ARG;
     return rl_launch_status();

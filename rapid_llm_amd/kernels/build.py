@@ -59,7 +59,7 @@ DEFAULT_HEAD_DIMS = tuple(range(16, 257, 16))
 
 # pairs of (key, value) head sizes of the tile attention that build_all() builds ahead of time
 DEFAULT_TILE_HEAD_DIMS = (
-    (16, 16), (16, 48), (32, 16), (32, 32), (48, 32), (64, 32), (64, 64), (64, 128), (96, 80), (128, 64), (128, 96),
+    (16, 16), (16, 32), (16, 48), (32, 16), (32, 32), (48, 32), (64, 32), (64, 64), (64, 128), (96, 80), (128, 64), (128, 96),
     (128, 128), (160, 144), (320, 256), (576, 512),
 )
 

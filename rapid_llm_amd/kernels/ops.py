@@ -192,7 +192,7 @@ def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, fed: Option
         core().rl_embed(
             _p(ids), _p(fed), 0 if fed is None else fed.numel(), _p(table), _tag(table.dtype), _p(out),
             tokens, hidden, vocab, ctypes.c_float(scale), _p(positions if with_positions else None),
-            _p(inv_freq), _p(pos_table), _stream(),
+            _p(inv_freq), _p(pos_table), 0 if pos_table is None else pos_table.shape[0], _stream(),
         ),
         "rl_embed",
     )

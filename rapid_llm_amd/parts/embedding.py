@@ -56,6 +56,7 @@ class TokenEmbedding(Embedding):
 
     def bind(self, params, runtime) -> None:
         self.table = params[self.name + ".weight"]
+        self.max_seq_len = int(runtime.max_seq_len)
         if self.position_table_name is not None:
             self.position_table = params[self.name + ".positions"]
             if self.position_table.dtype != self.table.dtype:  # one stored wider than the other
@@ -70,7 +71,9 @@ class TokenEmbedding(Embedding):
         """Rows of the table for the ids; an id ``-(r + 1)`` takes ``ctx.fed_tokens[r]``."""
         out = torch.empty((token_ids.numel(), self.hidden_size), dtype=torch.float32, device=token_ids.device)
         learned = self.position_table is not None
-        if learned and ctx.max_position >= self.positions:
+        # (a recorded step names the end of its context bucket, which may lie beyond the longest
+        # sequence the engine admits; no request's position does)
+        if learned and min(ctx.max_position, self.max_seq_len - 1) >= self.positions:
             raise ops.KernelError(f"position {ctx.max_position} is beyond the {self.positions} learned positions")
         ops.embed(token_ids, self.table, out, getattr(ctx, "fed_tokens", None), self.scale,
                   ctx.positions if (self.inv_freq is not None or learned) else None, self.inv_freq,

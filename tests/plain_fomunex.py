@@ -2,7 +2,9 @@
 the tests.  One function per mechanism, whole sequences only, no cache, no batching; it shares
 no code with the package.
 
-``cfg`` is the ``config.json`` dictionary, ``w`` maps checkpoint tensor names to tensors.
+``cfg`` is the ``config.json`` dictionary, ``w`` maps checkpoint tensor names to tensors.  ``cast``
+(optional) is applied wherever an engine that computes in a narrower type would round: the
+normed rows, the projections' results, the activations; never to what the design keeps in 32-bit.
 """
 
 from __future__ import annotations
@@ -23,10 +25,6 @@ def scalar_norm(x, g, eps):
     return rms(x, eps) * g
 
 
-def gelu_tanh(z):
-    return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z**3)))
-
-
 def silu(z):
     return z * torch.sigmoid(z)
 
@@ -40,14 +38,18 @@ def softplus(z):
 # --------------------------------------------------------------------------- #
 
 
-def attention(m: dict, w: dict, p: str, h: torch.Tensor, eps: float) -> torch.Tensor:
+def same(x):
+    return x
+
+
+def attention(m: dict, w: dict, p: str, h: torch.Tensor, eps: float, cast=same) -> torch.Tensor:
     T = h.shape[0]
     H, G, d = m["heads"], m.get("kv_heads") or m["heads"], m["dim"]
     dv = m.get("vdim") or d
-    q = (h @ w[p + "q"].T).view(T, H, d)
-    k = (h @ w[p + "k"].T).view(T, G, d)
-    v = (h @ w[p + "v"].T).view(T, G, dv)
-    q, k = rms(q, eps), rms(k, eps)
+    q = cast(h @ w[p + "q"].T).view(T, H, d)
+    k = cast(h @ w[p + "k"].T).view(T, G, d)
+    v = cast(h @ w[p + "v"].T).view(T, G, dv)
+    q, k = cast(rms(q, eps)), cast(rms(k, eps))
     cap = m.get("softcap")
     window = (m.get("mask") or {}).get("size") or 0
     i = torch.arange(T).view(T, 1)
@@ -67,10 +69,10 @@ def attention(m: dict, w: dict, p: str, h: torch.Tensor, eps: float) -> torch.Te
         e = torch.exp(s - top)
         den = e.sum(-1, keepdim=True) + torch.exp(sink - top)
         out[:, head] = (e / den) @ v[:, kv]
-    return out.reshape(T, H * dv) @ w[p + "o"].T
+    return cast(out.reshape(T, H * dv)) @ w[p + "o"].T
 
 
-def wkv(m: dict, w: dict, p: str, h: torch.Tensor, eps: float) -> torch.Tensor:
+def wkv(m: dict, w: dict, p: str, h: torch.Tensor, eps: float, cast=same) -> torch.Tensor:
     T = h.shape[0]
     H, d = m["heads"], m["dim"]
     prev = torch.cat([torch.zeros(1, h.shape[1], dtype=F), h[:-1]], 0)
@@ -78,10 +80,10 @@ def wkv(m: dict, w: dict, p: str, h: torch.Tensor, eps: float) -> torch.Tensor:
     def mix(s):
         return h + (prev - h) * w[p + "mu." + s]
 
-    r = (mix("r") @ w[p + "r"].T).view(T, H, d)
-    k = (mix("k") @ w[p + "k"].T).view(T, H, d)
-    v = (mix("v") @ w[p + "v"].T).view(T, H, d)
-    gate = silu(mix("g") @ w[p + "g"].T)
+    r = cast(cast(mix("r")) @ w[p + "r"].T).view(T, H, d)
+    k = cast(cast(mix("k")) @ w[p + "k"].T).view(T, H, d)
+    v = cast(cast(mix("v")) @ w[p + "v"].T).view(T, H, d)
+    gate = silu(cast(cast(mix("g")) @ w[p + "g"].T))
     decay = torch.exp(-torch.exp(torch.tanh(mix("w") @ w[p + "w1"].T) @ w[p + "w2"].T + w[p + "w0"])).view(T, H, d)
     u = w[p + "u"]  # [H, d]
     S = torch.zeros(H, d, d, dtype=F)  # [head, key channel, value channel]
@@ -91,17 +93,17 @@ def wkv(m: dict, w: dict, p: str, h: torch.Tensor, eps: float) -> torch.Tensor:
         out[t] = torch.einsum("hkv,hk->hv", S + u.unsqueeze(-1) * kv, r[t])
         S = decay[t].unsqueeze(-1) * S + kv
     out = rms(out, eps).reshape(T, H * d) * w[p + "norm"] * gate
-    return out @ w[p + "o"].T
+    return cast(out) @ w[p + "o"].T
 
 
-def mamba2(m: dict, w: dict, p: str, h: torch.Tensor, eps: float) -> torch.Tensor:
+def mamba2(m: dict, w: dict, p: str, h: torch.Tensor, eps: float, cast=same) -> torch.Tensor:
     T = h.shape[0]
     H, P, N, G = m["heads"], m["vdim"], m["state"], m["groups"]
     taps, parts = m["conv"], m["norm_groups"]
     inner = H * P
     zxbcdt = h @ w[p + "in"].T
-    z = zxbcdt[:, :inner]
-    xbc = zxbcdt[:, inner : 2 * inner + 2 * G * N]
+    z = cast(zxbcdt[:, :inner])
+    xbc = cast(zxbcdt[:, inner : 2 * inner + 2 * G * N])
     dt = zxbcdt[:, 2 * inner + 2 * G * N :]
     channels = xbc.shape[1]
     padded = torch.cat([torch.zeros(taps - 1, channels, dtype=F), xbc], 0)
@@ -124,7 +126,7 @@ def mamba2(m: dict, w: dict, p: str, h: torch.Tensor, eps: float) -> torch.Tenso
             out[t, head] = S[head].T @ C[t, g] + w[p + "D"][head] * x[t, head]
     y = out.reshape(T, inner) * silu(z)
     y = rms(y.view(T, parts, inner // parts), eps).reshape(T, inner) * w[p + "norm"]
-    return y @ w[p + "o"].T
+    return cast(y) @ w[p + "o"].T
 
 
 MIXERS = {"attention": attention, "wkv": wkv, "mamba2": mamba2}
@@ -135,20 +137,23 @@ MIXERS = {"attention": attention, "wkv": wkv, "mamba2": mamba2}
 # --------------------------------------------------------------------------- #
 
 
-def dense(f: dict, w: dict, p: str, h: torch.Tensor, eps: float) -> torch.Tensor:
-    z = h @ w[p + "up"].T
-    a, b, c, e = w[p + "act"]
-    act = a * rms(z, eps) + b * rms(z**2, eps) + c * rms(z**3, eps) + e
-    return act @ w[p + "down"].T
+def polynorm(z: torch.Tensor, coefficients: torch.Tensor, eps: float) -> torch.Tensor:
+    a, b, c, e = coefficients
+    return a * rms(z, eps) + b * rms(z**2, eps) + c * rms(z**3, eps) + e
 
 
-def expert(w: dict, p: str, h: torch.Tensor, limit: float) -> torch.Tensor:
-    g = torch.clamp(h @ w[p + "gate"].T, max=limit)
-    u = torch.clamp(h @ w[p + "up"].T, -limit, limit)
-    return (g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ w[p + "down"].T
+def dense(f: dict, w: dict, p: str, h: torch.Tensor, eps: float, cast=same) -> torch.Tensor:
+    z = cast(h @ w[p + "up"].T)
+    return cast(polynorm(z, w[p + "act"], eps)) @ w[p + "down"].T
 
 
-def moe(f: dict, w: dict, p: str, h: torch.Tensor, eps: float) -> torch.Tensor:
+def expert(w: dict, p: str, h: torch.Tensor, limit: float, cast=same) -> torch.Tensor:
+    g = torch.clamp(cast(h @ w[p + "gate"].T), max=limit)
+    u = torch.clamp(cast(h @ w[p + "up"].T), -limit, limit)
+    return cast(g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ w[p + "down"].T
+
+
+def moe(f: dict, w: dict, p: str, h: torch.Tensor, eps: float, cast=same) -> torch.Tensor:
     experts, top = f["router"]["experts"], f["router"]["top"]
     limit = f["expert"]["limit"]
     scores = torch.sigmoid(h @ w[p + "router"].T)
@@ -156,7 +161,7 @@ def moe(f: dict, w: dict, p: str, h: torch.Tensor, eps: float) -> torch.Tensor:
     for t in range(h.shape[0]):
         chosen = torch.topk(scores[t], top).indices
         for e in chosen.tolist():
-            out[t] += expert(w, f"{p}e{e}.", (scores[t, e] * h[t]).unsqueeze(0), limit)[0]
+            out[t] += expert(w, f"{p}e{e}.", (scores[t, e] * h[t]).unsqueeze(0), limit, cast)[0]
     return out
 
 
@@ -168,7 +173,7 @@ FEED_FORWARDS = {"dense": dense, "moe": moe}
 # --------------------------------------------------------------------------- #
 
 
-def forward(cfg: dict, w: dict, tokens: list[int], streams: list | None = None) -> torch.Tensor:
+def forward(cfg: dict, w: dict, tokens: list[int], streams: list | None = None, cast=same) -> torch.Tensor:
     """Logits ``[T, vocab]`` of one sequence from its start.  ``streams``: a list that receives
     the residual stream after every layer."""
     w = {name: t.to(F) for name, t in w.items()}
@@ -178,13 +183,13 @@ def forward(cfg: dict, w: dict, tokens: list[int], streams: list | None = None) 
     for i, layer in enumerate(cfg["layers"]):
         src = layer.get("weights_of")
         p = f"l{i if src is None else src}."
-        x = x + MIXERS[layer["type"]](layer["mixer"], w, p + "mix.", scalar_norm(x, w[p + "norm1"], eps), eps)
+        x = x + MIXERS[layer["type"]](layer["mixer"], w, p + "mix.", cast(scalar_norm(x, w[p + "norm1"], eps)), eps, cast)
         if layer.get("mlp") is not None:
             kind = layer["mlp"].get("kind", "dense")
-            x = x + FEED_FORWARDS[kind](layer["mlp"], w, p + "mlp.", scalar_norm(x, w[p + "norm2"], eps), eps)
+            x = x + FEED_FORWARDS[kind](layer["mlp"], w, p + "mlp.", cast(scalar_norm(x, w[p + "norm2"], eps)), eps, cast)
         if streams is not None:
             streams.append(x.clone())
-    x = scalar_norm(x, w["final.norm"], eps)
+    x = cast(scalar_norm(x, w["final.norm"], eps))
     logits = (x @ w["head"].T) * cfg["logit_scale"]
     cap = cfg.get("logit_softcap")
     if cap:

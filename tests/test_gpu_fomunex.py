@@ -1,0 +1,676 @@
+"""The Fomunex decoder in the engine against the plain implementation of ``plain_fomunex.py``:
+every mechanism alone, every way of cutting requests into steps, state slots and pages that are
+used again, the edges of windows and pages, long decoding, and greedy generation through the
+entry point."""
+
+import math
+import random
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+import parity
+import plain_fomunex as pf
+import replay_util as ru
+from fomunex_configs import (
+    BF16_ROWS_BEYOND,
+    BF16_TIMES_ROUNDING,
+    FOMU,
+    load_plain,
+    make_model_dir,
+    random_tokens,
+    row_errors,
+)
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+F32_ROW = 2e-4  # float32 rows against float64: root mean square over a row, relative to the logits' spread
+D64 = torch.float64
+
+
+def _ops():
+    from rapid_llm_amd.kernels import ops
+
+    return ops
+
+
+def bf16_round(t):
+    return t.bfloat16().to(t.dtype)
+
+
+def _tol(dtype, f32=2e-5, bf16=2e-2):
+    return dict(rtol=f32, atol=f32) if dtype == torch.float32 else dict(rtol=bf16, atol=bf16)
+
+
+def _step(lens, slots):
+    """What the recurrent kernels read of a step: the requests' offsets and their state rows."""
+    cu = [0]
+    for n in lens:
+        cu.append(cu[-1] + n)
+    return SimpleNamespace(
+        cu_seqlens=torch.tensor(cu, dtype=torch.int32, device=DEV),
+        seq_slots=torch.tensor(slots, dtype=torch.int32, device=DEV),
+        num_seqs=len(lens), h_seq_lens=list(lens), h_seq_slots=list(slots),
+    )
+
+
+def _cuts(total, sizes):
+    """``total`` tokens cut into portions of the given sizes in turn."""
+    out, at, i = [], 0, 0
+    while at < total:
+        n = min(sizes[i % len(sizes)], total - at)
+        out.append((at, at + n))
+        at += n
+        i += 1
+    return out
+
+
+# --------------------------------------------------------------------------- #
+# time mixing: the mixes with the token before, and the scan
+# --------------------------------------------------------------------------- #
+
+
+def _time_mixing_oracle(r, k, v, g, pre, bias, u, nw, eps):
+    """One request from a zero state, float64: ``[T, heads, d]`` operands."""
+    T, H, d = r.shape
+    w = torch.exp(-torch.exp(pre + bias))
+    S = torch.zeros(H, d, d, dtype=D64)
+    out = torch.zeros(T, H, d, dtype=D64)
+    for t in range(T):
+        kv = k[t].unsqueeze(-1) * v[t].unsqueeze(-2)
+        out[t] = ((S + u.unsqueeze(-1) * kv) * r[t].unsqueeze(-1)).sum(1)
+        S = w[t].unsqueeze(-1) * S + kv
+    out = out / torch.sqrt(out.square().mean(-1, keepdim=True) + eps)
+    return out * nw * (g * torch.sigmoid(g))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("heads,d", [(3, 16), (5, 20), (2, 64), (1, 100), (1, 200), (4, 1)])
+def test_time_mixing_scan_continues_from_the_slot(dtype, heads, d):
+    """Three requests in portions of changing size, down to one token, interleaved in shared
+    steps, on shuffled slots of which one is used again by a later request."""
+    ops = _ops()
+    gen = torch.Generator().manual_seed(heads * 100 + d)
+    eps, inner = 1e-5, heads * d
+    lengths = {"a": 37, "b": 5, "c": 64, "d": 9}
+    data, want = {}, {}
+    bias = torch.randn(inner, generator=gen) * 1.5 - 2.5
+    u = torch.randn(heads, d, generator=gen) * 0.5
+    nw = 1.0 + 0.1 * torch.randn(inner, generator=gen)
+    for rid, T in lengths.items():
+        r, k, v, g = (torch.randn(T, inner, generator=gen).to(dtype).float() for _ in range(4))
+        pre = torch.randn(T, inner, generator=gen)
+        data[rid] = (r, k, v, g, pre)
+        shape = (T, heads, d)
+        want[rid] = _time_mixing_oracle(
+            r.double().view(shape), k.double().view(shape), v.double().view(shape), g.double().view(shape),
+            pre.double().view(shape), bias.double().view(heads, d), u.double(), nw.double().view(heads, d), eps,
+        ).reshape(T, inner)
+    S = torch.full((5, heads, d, d), float("nan"), device=DEV)
+    slot = {"a": 3, "b": 0, "c": 1, "d": 0}  # d takes b's slot after b has ended
+    cuts = {"a": _cuts(37, (7, 1, 2, 11)), "b": _cuts(5, (2, 3)), "c": _cuts(64, (1, 1, 30, 2)), "d": _cuts(9, (9,))}
+    got = {rid: [] for rid in lengths}
+    live = ["a", "b", "c"]
+    while any(cuts[r] for r in lengths):
+        if not cuts["b"] and "d" not in live:
+            live = ["a", "d", "c"]
+        now = [r for r in live if cuts[r]]
+        spans = [cuts[r].pop(0) for r in now]
+        for r, (a, _b) in zip(now, spans):
+            if a == 0:
+                S[slot[r]].zero_()  # what taking a slot does
+        ctx = _step([b - a for a, b in spans], [slot[r] for r in now])
+        parts = [torch.cat([data[r][i][a:b] for r, (a, b) in zip(now, spans)]) for i in range(5)]
+        r_, k_, v_, g_ = (p.to(DEV, dtype) for p in parts[:4])
+        out = torch.empty_like(r_)
+        ops.wkv(r_, k_, v_, g_, parts[4].to(DEV), bias.to(DEV), u.to(DEV), nw.to(DEV), out, ctx, S, heads, d, eps)
+        at = 0
+        for r, (a, b) in zip(now, spans):
+            got[r].append(out[at : at + b - a].float().cpu())
+            at += b - a
+    for rid in lengths:
+        torch.testing.assert_close(torch.cat(got[rid]).double(), want[rid], **_tol(dtype, 5e-5, 3e-2))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("width", [96, 100, 7])
+def test_mixes_with_the_token_before(dtype, width):
+    ops = _ops()
+    gen = torch.Generator().manual_seed(width)
+    x = torch.randn(23, width, generator=gen).to(dtype)
+    mu = torch.rand(5 * width, generator=gen)
+    state = torch.randn(4, width, generator=gen)
+    lens, slots = [10, 1, 12], [2, 0, 3]
+    mixes = torch.empty((4, 23, width), dtype=dtype, device=DEV)
+    last = torch.empty((23, width), dtype=torch.float32, device=DEV)
+    st = state.clone().to(DEV)
+    ops.token_shift(x.to(DEV), mu.to(DEV), st, mixes, last, _step(lens, slots))
+    at = 0
+    for n, slot in zip(lens, slots):
+        h = x[at : at + n].double()
+        prev = torch.cat([state[slot : slot + 1].double(), h[:-1]])
+        for b in range(5):
+            want = h + (prev - h) * mu[b * width : (b + 1) * width].double()
+            have = (mixes[b, at : at + n] if b < 4 else last[at : at + n]).double().cpu()
+            torch.testing.assert_close(have, want, **_tol(dtype if b < 4 else torch.float32, 1e-6, 1e-2))
+        assert torch.equal(st[slot].cpu(), h[-1].float())
+        at += n
+    assert torch.equal(st[1].cpu(), state[1])  # a slot no request of the step holds
+
+
+# --------------------------------------------------------------------------- #
+# the state-space mixer: short convolution, scan, gate and grouped norm
+# --------------------------------------------------------------------------- #
+
+
+def _state_space_oracle(xbc, dt_raw, z, conv, conv_b, dt_bias, a_log, skip, heads, P, N, groups):
+    T, channels = xbc.shape
+    taps = conv.shape[1]
+    inner = heads * P
+    padded = torch.cat([torch.zeros(taps - 1, channels, dtype=D64), xbc])
+    y = conv_b.clone().expand(T, channels).clone()
+    for tap in range(taps):
+        y = y + padded[tap : tap + T] * conv[:, tap]
+    y = y * torch.sigmoid(y)
+    x, B, C = y[:, :inner].view(T, heads, P), y[:, inner : inner + groups * N].view(T, groups, N), \
+        y[:, inner + groups * N :].view(T, groups, N)
+    dt = torch.nn.functional.softplus(dt_raw + dt_bias)
+    S = torch.zeros(heads, N, P, dtype=D64)
+    out = torch.zeros(T, heads, P, dtype=D64)
+    for t in range(T):
+        for h in range(heads):
+            grp = h // (heads // groups)
+            S[h] = torch.exp(-torch.exp(a_log[h]) * dt[t, h]) * S[h] + dt[t, h] * torch.outer(B[t, grp], x[t, h])
+            out[t, h] = S[h].T @ C[t, grp] + skip[h] * x[t, h]
+    return y, out.reshape(T, inner) * (z * torch.sigmoid(z))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("heads,P,N,groups,taps", [(4, 16, 24, 2, 3), (6, 10, 12, 3, 2), (2, 64, 64, 1, 8), (1, 16, 1, 1, 1),
+                                                   (2, 32, 130, 2, 4), (3, 200, 8, 1, 4)])
+def test_convolution_and_state_space_scan_continue_from_the_slot(dtype, heads, P, N, groups, taps):
+    """Portions shorter than the convolution's reach (one, two and three tokens in a row), so that
+    the kept inputs are shifted and not replaced; two requests in shared steps."""
+    ops = _ops()
+    gen = torch.Generator().manual_seed(heads * 1000 + P + N)
+    inner = heads * P
+    channels = inner + 2 * groups * N
+    width = inner + channels + 3  # columns beyond the packed ones are not this kernel's
+    conv, conv_b = torch.randn(channels, taps, generator=gen) * 0.6, torch.randn(channels, generator=gen) * 0.2
+    dt_bias, a_log = torch.randn(heads, generator=gen) - 1.0, torch.randn(heads, generator=gen) - 1.0
+    skip = 1.0 + 0.3 * torch.randn(heads, generator=gen)
+    lengths = {"a": 41, "b": 18}
+    data, want = {}, {}
+    for rid, T in lengths.items():
+        packed = torch.randn(T, width, generator=gen).to(dtype).float()
+        dt_raw = torch.randn(T, heads, generator=gen)
+        data[rid] = (packed, dt_raw)
+        want[rid] = _state_space_oracle(
+            packed[:, inner : inner + channels].double(), dt_raw.double(), packed[:, :inner].double(), conv.double(),
+            conv_b.double(), dt_bias.double(), a_log.double(), skip.double(), heads, P, N, groups)
+    conv_state = torch.zeros((3, max(taps - 1, 1), channels), device=DEV)
+    S = torch.zeros((3, heads, N, P), device=DEV)
+    slot = {"a": 2, "b": 0}
+    cuts = {"a": _cuts(41, (1, 1, 2, 1, 3, 9, 2)), "b": _cuts(18, (2, 1, 1, 1, 7))}
+    got = {rid: ([], []) for rid in lengths}
+    while any(cuts.values()):
+        now = [r for r in lengths if cuts[r]]
+        spans = [cuts[r].pop(0) for r in now]
+        ctx = _step([b - a for a, b in spans], [slot[r] for r in now])
+        packed = torch.cat([data[r][0][a:b] for r, (a, b) in zip(now, spans)]).to(DEV, dtype)
+        dt_raw = torch.cat([data[r][1][a:b] for r, (a, b) in zip(now, spans)]).to(DEV)
+        mixed = torch.empty((packed.shape[0], channels), dtype=torch.float32, device=DEV)
+        ops.causal_conv(packed, inner, conv.to(DEV), conv_b.to(DEV), conv_state, mixed, ctx)
+        out = torch.empty((packed.shape[0], inner), dtype=torch.float32, device=DEV)
+        ops.state_space_scan(mixed, dt_raw, dt_bias.to(DEV), a_log.to(DEV), skip.to(DEV), packed, out, ctx, S,
+                             heads, P, N, groups)
+        at = 0
+        for r, (a, b) in zip(now, spans):
+            got[r][0].append(mixed[at : at + b - a].cpu())
+            got[r][1].append(out[at : at + b - a].cpu())
+            at += b - a
+    for rid in lengths:
+        torch.testing.assert_close(torch.cat(got[rid][0]).double(), want[rid][0], rtol=2e-5, atol=2e-5)
+        torch.testing.assert_close(torch.cat(got[rid][1]).double(), want[rid][1], rtol=2e-4, atol=2e-4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("width,parts", [(64, 4), (60, 5), (128, 1), (18, 18), (2000, 2)])
+def test_norm_in_equal_parts(dtype, width, parts):
+    ops = _ops()
+    y = torch.randn(9, width) * 3.0
+    w = 1.0 + 0.2 * torch.randn(width)
+    out = torch.empty((9, width), dtype=dtype, device=DEV)
+    ops.group_rmsnorm(y.to(DEV), w.to(DEV), out, parts, 1e-5)
+    want = pf.rms(y.double().view(9, parts, width // parts), 1e-5).reshape(9, width) * w.double()
+    torch.testing.assert_close(out.double().cpu(), want, **_tol(dtype, 1e-5, 1e-2))
+
+
+# --------------------------------------------------------------------------- #
+# feed-forward pieces, the two ends
+# --------------------------------------------------------------------------- #
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("cols", [80, 50, 7, 3000])
+def test_polynomial_activation_over_normalised_powers(dtype, cols):
+    ops = _ops()
+    z = (torch.randn(11, cols) * 2.0).to(dtype)
+    coef = torch.tensor([0.7, -0.4, 1.3, 0.25])
+    out = torch.empty_like(z, device=DEV)
+    ops.polynorm(z.to(DEV), out, coef.to(DEV), 1e-5)
+    want = pf.polynorm(z.double(), coef.double(), 1e-5)
+    torch.testing.assert_close(out.double().cpu(), want, **_tol(dtype, 2e-5, 3e-2))
+    alone = torch.empty((1, cols), dtype=dtype, device=DEV)
+    ops.polynorm(z[4:5].contiguous().to(DEV), alone, coef.to(DEV), 1e-5)
+    assert torch.equal(alone[0], out[4])  # a row does not depend on the rest of the step
+
+
+@pytest.mark.parametrize("experts,top", [(6, 2), (3, 1), (4, 4), (70, 5), (1, 1)])
+def test_router_with_sigmoid_scores_taken_as_they_are(experts, top):
+    ops = _ops()
+    h = torch.randn(33, 48)
+    w = torch.randn(experts, 48) * 0.8
+    got = ops.router(h.to(DEV), w.to(DEV), top, 1.0, None, "sigmoid").cpu()
+    scores = torch.sigmoid(h.double() @ w.double().T)
+    for t in range(33):
+        chosen = set(torch.topk(scores[t], top).indices.tolist())
+        assert set(torch.nonzero(got[t]).flatten().tolist()) == chosen
+        for e in chosen:
+            assert abs(float(got[t, e]) - float(scores[t, e])) < 1e-5
+    bf = ops.router(h.bfloat16().to(DEV), w.to(DEV), top, 1.0, None, "sigmoid").cpu()
+    torch.testing.assert_close(bf.sum(1), torch.sigmoid(h.bfloat16().double() @ w.double().T).topk(top).values.sum(1).float(),
+                               rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("experts,ff,limit", [(5, 27, 1.5), (6, 24, 2.0), (1, 16, 0.5)])
+def test_an_experts_weight_scales_what_it_reads(dtype, experts, ff, limit):
+    ops = _ops()
+    gate_up = (torch.randn(13, 2 * experts * ff) * 2.0).to(dtype)
+    route = torch.rand(13, experts)
+    route[route < 0.5] = 0.0
+    out = torch.empty((13, experts * ff), dtype=dtype, device=DEV)
+    ops.swiglu(gate_up.to(DEV), out, limit, 1.702, route=route.to(DEV), expert_ff=ff, route_input=True)
+    f = route.double().repeat_interleave(ff, 1)
+    g = torch.clamp(gate_up[:, : experts * ff].double() * f, max=limit)
+    u = torch.clamp(gate_up[:, experts * ff :].double() * f, -limit, limit)
+    want = g * torch.sigmoid(1.702 * g) * (u + 1.0)
+    torch.testing.assert_close(out.double().cpu(), want, **_tol(dtype, 1e-5, 2e-2))
+    assert float(out.double().cpu()[f == 0].abs().max() if (f == 0).any() else 0.0) == 0.0  # an unused expert adds nothing
+
+
+def test_logits_scaled_then_capped():
+    ops = _ops()
+    v = torch.randn(5, 97) * 40.0
+    got = v.clone().to(DEV)
+    ops.scale_cap(got, 0.5, 30.0)
+    torch.testing.assert_close(got.cpu().double(), 30.0 * torch.tanh(v.double() * 0.5 / 30.0), rtol=1e-5, atol=1e-5)
+    got = v.clone().to(DEV)
+    ops.scale_cap(got, 1.3, 0.0)
+    torch.testing.assert_close(got.cpu(), v * 1.3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("hidden", [96, 100])
+def test_embedding_with_learned_position_vectors(dtype, hidden):
+    ops = _ops()
+    table, pos = torch.randn(50, hidden).to(dtype), torch.randn(30, hidden).to(dtype)
+    ids = torch.tensor([3, 49, 0, 7], dtype=torch.int32)
+    positions = torch.tensor([0, 29, 5, 6], dtype=torch.int32)
+    out = torch.empty((4, hidden), dtype=torch.float32, device=DEV)
+    ops.embed(ids.to(DEV), table.to(DEV), out, None, 1.0, positions.to(DEV), None, pos.to(DEV))
+    want = table.float()[ids.long()] + pos.float()[positions.long()]
+    torch.testing.assert_close(out.cpu(), want, rtol=1e-6, atol=1e-6)
+
+
+# --------------------------------------------------------------------------- #
+# attention: capped scores, a distance term per head, a learned sink, a window
+# --------------------------------------------------------------------------- #
+
+
+def _attention_oracle(q, k, v, scale, window, cap, slopes, sink, first_row):
+    """The last ``q.shape[0]`` positions of one request: ``q [n, H, d]``, ``k [t, G, d]``, ``v [t, G, dv]``."""
+    t, n, H, G = k.shape[0], q.shape[0], q.shape[1], k.shape[1]
+    i = torch.arange(first_row, first_row + n).view(n, 1)
+    j = torch.arange(t).view(1, t)
+    seen = (j <= i) & ((i - j < window) if window else (j >= 0))
+    out = torch.zeros(n, H, v.shape[2], dtype=D64)
+    for h in range(H):
+        g = h // (H // G)
+        s = (q[:, h].double() @ k[:, g].double().T) * scale
+        if cap:
+            s = cap * torch.tanh(s / cap)
+        if slopes is not None:
+            s = s - slopes[h].double() * (i - j)
+        s = s.masked_fill(~seen, -math.inf)
+        top = torch.maximum(s.max(1, keepdim=True).values, sink[h].double())
+        e = torch.exp(s - top)
+        out[:, h] = (e / (e.sum(1, keepdim=True) + torch.exp(sink[h].double() - top))) @ v[:, g].double()
+    return out.reshape(n, -1)
+
+
+def _paged(seqs, H, G, d, dv, page, dtype, seed, window, scale, cap, slopes, sink, spike=None):
+    """``seqs`` = (tokens already cached, tokens of this step) per request, on shuffled pages and
+    slots; what no query may read is NaN (unwritten slots of a page, pages the window has passed)."""
+    rng = random.Random(seed)
+    gen = torch.Generator().manual_seed(seed)
+    total = sum(-(-(a + n) // page) for a, n in seqs) + 1
+    free = list(range(1, total))
+    rng.shuffle(free)
+    table = torch.zeros((len(seqs) + 2, max(-(-(a + n) // page) for a, n in seqs) + 1), dtype=torch.int32)
+    kc = torch.full((total, G, page, d), float("nan"))
+    vc = torch.full((total, G, dv, page), float("nan"))
+    slots = list(range(len(seqs) + 2))
+    rng.shuffle(slots)
+    rows, positions, token_slot, want = [], [], [], []
+    for i, (a, n) in enumerate(seqs):
+        t = a + n
+        k, v, q = torch.randn(t, G, d, generator=gen), torch.randn(t, G, dv, generator=gen), torch.randn(n, H, d, generator=gen)
+        k, q = (x / x.square().mean(-1, keepdim=True).sqrt() for x in (k, q))  # as the head norm leaves them
+        if spike is not None and spike[0] == i:
+            # one key matches the request's last query in every head, far beyond every other score
+            far = spike[1]
+            q[-1] = q[-1, 0]
+            k[far] = q[-1, 0] * 4.0
+            v[far] = 7.0
+        if dtype == torch.bfloat16:
+            q, k, v = (x.bfloat16().float() for x in (q, k, v))
+        first_needed = max(0, a - window + 1) // page if window else 0
+        for p in range(-(-t // page)):
+            pid = free.pop()
+            if p < first_needed:
+                continue  # given back: the table names the null page there
+            table[slots[i], p] = pid
+            lo, hi = p * page, min(t, (p + 1) * page)
+            kc[pid, :, : hi - lo] = k[lo:hi].transpose(0, 1)
+            vc[pid, :, :, : hi - lo] = v[lo:hi].permute(1, 2, 0)
+        want.append(_attention_oracle(q, k, v, scale, window, cap, slopes, sink, a))
+        rows.append(q.reshape(n, H * d))
+        positions += list(range(a, t))
+        token_slot += [slots[i]] * n
+    ctx = SimpleNamespace(
+        positions=torch.tensor(positions, dtype=torch.int32, device=DEV),
+        token_slot=torch.tensor(token_slot, dtype=torch.int32, device=DEV),
+        token_ids=torch.zeros(len(positions), dtype=torch.int32, device=DEV),
+        h_seq_starts=[a for a, _ in seqs], h_seq_lens=[n for _, n in seqs], max_position=max(positions), extra={},
+    )
+    return torch.cat(rows).to(DEV, dtype), kc.to(DEV, dtype), vc.to(DEV, dtype), table.to(DEV), ctx, torch.cat(want)
+
+
+def _slopes(H, exponent=8.0):
+    return torch.exp2(-exponent * torch.arange(1, H + 1, dtype=D64) / H).float()
+
+
+def _run_attention(case, dtype, spike=None, seed=5):
+    ops = _ops()
+    H, G, d, dv, page, window, cap, seqs = case
+    sink = 2.0 + 1.5 * torch.randn(H, generator=torch.Generator().manual_seed(seed))
+    slopes = _slopes(H)
+    scale = 3.0 / d  # unit-norm heads: |q . k| <= d
+    q, kc, vc, table, ctx, want = _paged(seqs, H, G, d, dv, page, dtype, seed, window, scale, cap, slopes, sink, spike)
+    out = torch.empty((q.shape[0], H * dv), dtype=dtype, device=DEV)
+    ops.paged_attention(q, kc, vc, out, ctx, table, page, H, G, d, window, scale, value_dim=dv,
+                        sink_values=sink.to(DEV), score_cap=cap, slopes=slopes.to(DEV))
+    return out.double().cpu(), want
+
+
+ATTENTION_CASES = [
+    # H, G, d, dv, page, window, cap, (cached, new) per request
+    (4, 2, 16, 32, 8, 19, 8.0, [(0, 60), (45, 1), (200, 1), (30, 31), (0, 1), (18, 1), (19, 1)]),
+    (6, 3, 24, 10, 8, 33, 15.0, [(0, 50), (32, 1), (33, 1), (100, 2)]),          # sizes off the grid of 16
+    (8, 2, 64, 32, 16, 70, 40.0, [(300, 1), (5, 70), (0, 2), (69, 1), (70, 1)]),
+    (1, 1, 16, 16, 4, 0, 0.0, [(0, 40), (120, 1), (39, 3)]),                      # every key, no cap
+    (2, 2, 16, 16, 4, 1, 50.0, [(0, 9), (5, 1)]),                                 # a window of the own key alone
+    (3, 1, 12, 22, 4, 9, 0.0, [(0, 30), (8, 1), (9, 1), (50, 1)]),
+    (4, 1, 128, 64, 16, 600, 30.0, [(2000, 1), (590, 30), (0, 700)]),             # long contexts
+]
+
+
+@pytest.mark.parametrize("case", ATTENTION_CASES, ids=lambda c: f"h{c[0]}kv{c[1]}d{c[2]}v{c[3]}p{c[4]}w{c[5]}")
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_attention_with_cap_distance_term_and_learned_sink(case, dtype):
+    got, want = _run_attention(case, dtype)
+    torch.testing.assert_close(got, want, **_tol(dtype, 2e-5, 3e-2))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("d,dv,page", [(64, 32, 16), (16, 32, 8), (24, 10, 8)])
+def test_one_key_holds_the_mass_at_every_edge(dtype, d, dv, page):
+    """The last query's weight lies on one key: the last one inside the window, the first one
+    outside, the first and last of a page, the query's own; in a prompt's portion and decoded
+    alone.  The value of that key is 7 in every channel, every other value is of order one."""
+    H, G, window, cap = 4, 2, 41, 60.0
+    for cached, new in ((100, 1), (70, 31), (0, 101)):
+        last = cached + new - 1
+        for far, inside in ((last - window + 1, True), (last - window, False), (last, True),
+                            (last - last % page, True), (last - last % page - 1, True), (last - window + 2, True)):
+            case = (H, G, d, dv, page, window, cap, [(3, 2), (cached, new), (50, 1)])
+            got, want = _run_attention(case, dtype, spike=(1, far), seed=far + 3)
+            row = 2 + new - 1
+            torch.testing.assert_close(got, want, **_tol(dtype, 3e-5, 4e-2))
+            # the first head's distance term (a quarter a position) outweighs the key at the
+            # window's far end; the last head's hardly counts
+            tail = got[row].view(H, dv)[-1]
+            assert (float(tail.min()) > 6.0) == inside, (cached, new, far)
+
+
+# --------------------------------------------------------------------------- #
+# the model through the engine's step function
+# --------------------------------------------------------------------------- #
+LENGTHS = {
+    "A": [1, 2, 3, 18, 19, 20, 21, 40, 57, 130],  # the first tokens; around the window of 19 and pages of 8
+    "B": [1, 2, 4, 5, 9, 33, 80],
+    "C": [1, 2, 8, 9, 10, 32, 33, 34, 35, 90],   # around the windows of 9 and 33
+    "D": [2, 15, 69, 70, 71, 72, 150],           # around the window of 70
+}
+
+
+def _requests(which):
+    cfg, _page, seed = FOMU[which]
+    return {f"q{i}": random_tokens(n, cfg["vocab"], seed * 100 + i) for i, n in enumerate(LENGTHS[which])}
+
+
+def _oracles(pcfg, pw, requests):
+    """Per request the plain logits in float64, and what rounding alone does to the rows of the
+    plain implementation with rounded activations: their median error and the error that nine rows
+    in ten stay under."""
+    want = {rid: pf.forward(pcfg, pw, toks) for rid, toks in requests.items()}
+    rounded = {rid: pf.forward(pcfg, pw, toks, cast=bf16_round) for rid, toks in requests.items()}
+    order = sorted(want)
+    rows = row_errors(torch.cat([rounded[r] for r in order]), torch.cat([want[r] for r in order]))
+    return want, (float(rows.median()), float(rows.quantile(0.9)))
+
+
+def _runner(model_dir, dtype, page, num_pages, max_seq_len, slots=4):
+    from rapid_llm_amd import EngineConfig, ModelRunner
+
+    runner = ModelRunner(
+        model_dir,
+        EngineConfig(dtype=dtype, max_seq_len=max_seq_len, page_size=page, num_pages=num_pages,
+                     max_num_seqs=slots, use_graph=False),
+    )
+    for layer in runner.device_cache.layers:  # whatever is read before it is written shows
+        for t in layer.pages.values() if layer.owns_pages else ():
+            t.fill_(float("nan"))
+    return runner
+
+
+def _check(got, want, dtype, label, rounding=None):
+    """float32: every row within the bound.  bfloat16: rounding moves most rows a little and a few
+    rows a lot (a token whose two best experts' scores lie closer than rounding moves them takes
+    another expert, in an engine as in the plain implementation with rounded activations, though
+    not at the same tokens; the recurrent states then carry the difference into later rows), so
+    the engine's typical rows are compared with the rounded plain implementation's typical rows,
+    and the rows far out may be a tenth of all."""
+    order = sorted(want)
+    if dtype == "bfloat16":
+        a, b = torch.cat([got[r] for r in order]), torch.cat([want[r] for r in order])
+        assert a.shape == b.shape and torch.isfinite(a).all(), label
+        rows = row_errors(a, b)
+        median, ninth = rounding
+        parity.record(label, float(rows.max()), float((a.double() - b.double()).abs().max() / b.double().std()))
+        assert float(rows.median()) <= BF16_TIMES_ROUNDING * median, (
+            f"{label}: half of the rows are off by more than {float(rows.median()):.4f} of the logits' spread, "
+            f"{BF16_TIMES_ROUNDING} times what rounding does to half of them ({median:.4f})")
+        beyond = rows > BF16_TIMES_ROUNDING * ninth
+        assert float(beyond.double().mean()) <= BF16_ROWS_BEYOND, (
+            f"{label}: {int(beyond.sum())} of {rows.numel()} rows are off by more than {BF16_TIMES_ROUNDING} times "
+            f"what rounding does to nine rows in ten ({ninth:.4f} of the logits' spread); the first is row "
+            f"{int(torch.nonzero(beyond)[0])}")
+        return
+    spread = float(torch.cat([want[r] for r in order]).double().std())
+    for rid in order:
+        assert got[rid].shape == want[rid].shape and torch.isfinite(got[rid]).all(), (label, rid)
+        rows = (got[rid].double() - want[rid].double()).square().mean(dim=1).sqrt() / spread
+        bad = rows > F32_ROW
+        assert not bad.any(), (
+            f"{label}: request {rid}, first wrong position {int(torch.nonzero(bad)[0])}, "
+            f"worst row {float(rows.max()):.3e} of the spread"
+        )
+
+
+@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_every_cut_matches_plain(tmp_path, which, dtype):
+    cfg, page, seed = FOMU[which]
+    model_dir = make_model_dir(tmp_path, which, sharp=3.0)
+    pcfg, pw = load_plain(model_dir)
+    requests = _requests(which)
+    want, rounding = _oracles(pcfg, pw, requests)
+    longest = max(LENGTHS[which])
+    schedules = {
+        "whole": ru.whole(requests),
+        "decode": ru.prefill_then_decode(requests, 50),
+        "token_by_token": ru.prefill_then_decode(requests, 10 ** 6),
+        "portions": ru.changing_portions(requests),
+        "portions_of_two": ru.changing_portions(requests, sizes=(2, 2, 3, 2, 64, 2)),
+        "mixed": ru.mixed(requests, seed, max_tokens=None),
+        "mixed_tight": ru.mixed(requests, seed + 1, max_tokens=2 * 64 * ((longest + 63) // 64)),
+    }
+    first = None
+    for label, steps in schedules.items():
+        pages = ru.pages_for(steps, requests, page) + 1
+        runner = _runner(model_dir, dtype, page, pages + 1, longest + 8)
+        got = ru.run_in_process(runner, steps)
+        _check(got, want, dtype, f"{which}/{dtype}/{label}", rounding)
+        if dtype == "float32":
+            # one order of summation however the requests are cut: the same bits
+            if first is None:
+                first = got
+            else:
+                for rid in got:
+                    assert torch.equal(got[rid], first[rid]), (label, rid)
+        runner.cache.check_invariants()
+        assert not runner.cache.live_requests()
+        del runner
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_batch_of_unequal_requests_equals_each_alone(tmp_path, dtype):
+    """One step holds a long prompt, a short one, a single first token and decoded tokens of two
+    requests at different depths; every row equals the row of the request run alone."""
+    which = "A"
+    cfg, page, seed = FOMU[which]
+    model_dir = make_model_dir(tmp_path, which, sharp=3.0)
+    requests = {f"u{i}": random_tokens(n, cfg["vocab"], 70 + i) for i, n in enumerate((90, 5, 1, 61, 30))}
+    runner = _runner(model_dir, dtype, page, 60, 100, slots=5)
+    alone = ru.run_in_process(runner, ru.whole(requests))
+    full = lambda r, a, b: {"id": r, "tokens": requests[r][a:b], "want": list(range(b - a))}  # noqa: E731
+    steps = [
+        {"step": 0, "entries": [full("u3", 0, 60), full("u4", 0, 29)], "end": []},
+        {"step": 1, "entries": [full("u0", 0, 90), full("u3", 60, 61), full("u1", 0, 5), full("u2", 0, 1), full("u4", 29, 30)],
+         "end": ["u0", "u1", "u2", "u3", "u4"]},
+    ]
+    got = ru.run_in_process(runner, steps)
+    for rid in requests:
+        if dtype == "float32":
+            assert torch.equal(got[rid], alone[rid]), rid
+        else:
+            assert float(row_errors(got[rid], alone[rid]).max()) < 0.1, rid
+    runner.cache.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_and_slots_used_again(tmp_path, dtype):
+    """Five requests through two slots, each a short prompt and then 200 tokens one by one, two at
+    a time in a step: the window passes over decoded tokens, its pages come back and are taken
+    again, and a later request finds the states of its slot zeroed."""
+    which = "A"
+    cfg, page, seed = FOMU[which]
+    model_dir = make_model_dir(tmp_path, which, sharp=3.0)
+    pcfg, pw = load_plain(model_dir)
+    requests = {f"d{i}": random_tokens(200 + 7 * i, cfg["vocab"], 40 + i) for i in range(5)}
+    want, rounding = _oracles(pcfg, pw, requests)
+    steps = ru.mixed(requests, 3, max_live=2, tail=195)
+    runner = _runner(model_dir, dtype, page, 2 * (-(-240 // page) + 1) + 2, 240, slots=2)
+    got = ru.run_in_process(runner, steps)
+    _check(got, want, dtype, f"long decoding/{dtype}", rounding)
+    runner.cache.check_invariants()
+
+
+def test_a_far_token_still_counts_through_the_states(tmp_path):
+    """A different first token changes the logits 150 positions later, far beyond every window:
+    only the recurrent states carry it; and it does so alike whether the tokens in between came
+    in one prompt or one by one."""
+    which = "A"
+    cfg, page, seed = FOMU[which]
+    model_dir = make_model_dir(tmp_path, which)
+    pcfg, pw = load_plain(model_dir)
+    toks = random_tokens(150, cfg["vocab"], 12)
+    other = [(toks[0] + 1) % cfg["vocab"]] + toks[1:]
+    want = {"same": pf.forward(pcfg, pw, toks), "other": pf.forward(pcfg, pw, other)}
+    assert float(row_errors(want["other"][-1:], want["same"][-1:]).max()) > 100 * F32_ROW
+    for steps_of in (ru.whole, lambda r: ru.prefill_then_decode(r, 140)):
+        runner = _runner(model_dir, "float32", page, 60, 160)
+        got = ru.run_in_process(runner, steps_of({"same": toks, "other": other}))
+        _check(got, want, "float32", "far token")
+
+
+def test_trace_program(tmp_path):
+    """``bin/trace_run`` as a child process on a mixed trace over a tight pool."""
+    which = "B"
+    cfg, page, seed = FOMU[which]
+    model_dir = make_model_dir(tmp_path, which, sharp=3.0)
+    pcfg, pw = load_plain(model_dir)
+    requests = _requests(which)
+    want, _rounding = _oracles(pcfg, pw, requests)
+    steps = ru.mixed(requests, seed + 5, max_tokens=256)
+    got = ru.run_trace_program(model_dir, "float32", steps, tmp_path / "out", 256, cfg["vocab"])
+    _check(got, want, "float32", "trace_run")
+
+
+@pytest.mark.parametrize("use_graph", [False, True])
+@pytest.mark.parametrize("which,dtype", [("A", "float32"), ("C", "float32"), ("D", "bfloat16")])
+def test_greedy_generation_through_the_entry_point(tmp_path, which, dtype, use_graph):
+    """``LLM.generate``: scheduler, chunked prompts beside decoding requests, sampling kernels;
+    decode steps eagerly and replayed from graphs.  The plain implementation re-runs the whole
+    sequence for every token; a bfloat16 engine may pick another of several nearly equal maxima."""
+    from rapid_llm_amd import LLM, SamplingParams
+
+    cfg, page, seed = FOMU[which]
+    model_dir = make_model_dir(tmp_path, which)
+    pcfg, pw = load_plain(model_dir)
+    prompts = [random_tokens(n, cfg["vocab"], seed + n) for n in (1, 7, 30, 45)]
+    llm = LLM(str(model_dir), dtype=dtype, page_size=page, num_pages=60, max_num_seqs=3, max_seq_len=96,
+              max_chunk_size=16, max_num_batched_tokens=32, use_cuda_graph=use_graph)
+    outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_gen_len=24))
+    gaps = []
+    for prompt, out in zip(prompts, outs):
+        ids = list(prompt)
+        for tok in out.token_ids:
+            logits = pf.forward(pcfg, pw, ids)[-1]
+            if dtype == "float32":
+                assert float(logits.max() - logits[tok]) <= 1e-3, (len(prompt), len(ids))
+            gaps.append(float(logits.max() - logits[tok]) / float(logits.std()))
+            ids.append(tok)
+        assert len(out.token_ids) == 24
+    if dtype == "bfloat16":
+        # most tokens are the plain choice; where rounding flipped an expert the engine's row may
+        # be another row altogether, and so its choice
+        gaps.sort()
+        assert gaps[len(gaps) // 2] <= 0.05 and gaps[int(0.85 * len(gaps))] <= 0.5, gaps[-10:]
+    llm.scheduler.cache.check_invariants()
+    assert not llm.scheduler.cache.live_requests()
