@@ -728,7 +728,7 @@ def _time_fomunex_kernels(z: dict, prompt_len: int, batch: int) -> dict:
     hs, P, N, G, taps = 2 * width // 64, 64, 128, 8, 4
     inner = hs * P
     channels = inner + 2 * G * N
-    S2 = torch.zeros((batch + 1, hs, N, P), device=dev)
+    S2 = torch.zeros((batch + 1, hs, P, N), device=dev)
     conv_state = torch.zeros((batch + 1, taps - 1, channels), device=dev)
     conv_w, conv_b = torch.randn(channels, taps, device=dev) * 0.5, torch.zeros(channels, device=dev)
     for what, lens in (("prefill", [prompt_len]), ("decode", [1] * batch)):

@@ -1517,30 +1517,67 @@ extern "C" int rl_read_buffer(const void* src, size_t bytes, unsigned* sink, int
 // powers element by element, (a, b, c, e) = coef[0..3].  One workgroup a row; the three sums of
 // squares and the result are float32, and a row's sums are formed in one order whatever the step.
 // --------------------------------------------------------------------------- //
-template <typename T>
+// three block-wide sums with one pair of barriers; `scratch` is a __shared__ float[48]
+__device__ inline void block_sum3(float& a, float& b, float& c, float* scratch) {
+    const int lane = threadIdx.x & (RL_WAVE - 1);
+    const int wave = threadIdx.x / RL_WAVE;
+    const int nwaves = (blockDim.x + RL_WAVE - 1) / RL_WAVE;
+    a = wave_sum(a);
+    b = wave_sum(b);
+    c = wave_sum(c);
+    __syncthreads();
+    if (lane == 0) {
+        scratch[wave] = a;
+        scratch[16 + wave] = b;
+        scratch[32 + wave] = c;
+    }
+    __syncthreads();
+    a = b = c = 0.f;
+    for (int i = 0; i < nwaves; ++i) {
+        a += scratch[i];
+        b += scratch[16 + i];
+        c += scratch[32 + i];
+    }
+}
+
+// VEC elements a thread and round (8 where the row allows 16-byte accesses, else 1)
+template <typename T, int VEC>
 __global__ __launch_bounds__(256) void polynorm_kernel(const T* __restrict__ x, T* __restrict__ out, int cols,
                                                        const float* __restrict__ coef, float eps) {
-    __shared__ float scratch[16];
+    struct alignas(sizeof(T) * VEC) Pack {
+        T v[VEC];
+    };
+    __shared__ float scratch[48];
     const T* row = x + (size_t)blockIdx.x * cols;
     T* dst = out + (size_t)blockIdx.x * cols;
     float s2 = 0.f, s4 = 0.f, s6 = 0.f;
-    for (int i = threadIdx.x; i < cols; i += blockDim.x) {
-        const float z = to_float(row[i]);
-        const float z2 = z * z;
-        s2 += z2;
-        s4 += z2 * z2;
-        s6 += z2 * z2 * z2;
+#pragma unroll 4
+    for (int i = VEC * threadIdx.x; i < cols; i += VEC * blockDim.x) {
+        const Pack in = *reinterpret_cast<const Pack*>(row + i);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            const float z = to_float(in.v[e]);
+            const float z2 = z * z;
+            s2 += z2;
+            s4 += z2 * z2;
+            s6 += z2 * z2 * z2;
+        }
     }
-    s2 = block_sum(s2, scratch);
-    s4 = block_sum(s4, scratch);
-    s6 = block_sum(s6, scratch);
+    block_sum3(s2, s4, s6, scratch);
     const float r1 = coef[0] * rsqrtf(s2 / (float)cols + eps);
     const float r2 = coef[1] * rsqrtf(s4 / (float)cols + eps);
     const float r3 = coef[2] * rsqrtf(s6 / (float)cols + eps);
-    const float e = coef[3];
-    for (int i = threadIdx.x; i < cols; i += blockDim.x) {
-        const float z = to_float(row[i]);
-        dst[i] = from_float<T>(z * r1 + (z * z) * r2 + (z * z * z) * r3 + e);
+    const float e0 = coef[3];
+#pragma unroll 4
+    for (int i = VEC * threadIdx.x; i < cols; i += VEC * blockDim.x) {
+        const Pack in = *reinterpret_cast<const Pack*>(row + i);
+        Pack o;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            const float z = to_float(in.v[e]);
+            o.v[e] = from_float<T>(z * r1 + (z * z) * r2 + (z * z * z) * r3 + e0);
+        }
+        *reinterpret_cast<Pack*>(dst + i) = o;
     }
 }
 
@@ -1548,11 +1585,18 @@ extern "C" int rl_polynorm(const void* x, void* out, int tokens, int cols, const
                            int act_type, hipStream_t stream) {
     if (tokens <= 0) return RL_OK;
     if (cols < 1 || !coef) return RL_ERR_ARG;
-    if (act_type == RL_F32)
-        hipLaunchKernelGGL(polynorm_kernel<float>, dim3(tokens), dim3(256), 0, stream, (const float*)x, (float*)out,
-                           cols, coef, eps);
+    const bool vec = cols % 8 == 0;
+    if (act_type == RL_F32 && vec)
+        hipLaunchKernelGGL((polynorm_kernel<float, 8>), dim3(tokens), dim3(256), 0, stream, (const float*)x,
+                           (float*)out, cols, coef, eps);
+    else if (act_type == RL_F32)
+        hipLaunchKernelGGL((polynorm_kernel<float, 1>), dim3(tokens), dim3(256), 0, stream, (const float*)x,
+                           (float*)out, cols, coef, eps);
+    else if (act_type == RL_BF16 && vec)
+        hipLaunchKernelGGL((polynorm_kernel<bf16_t, 8>), dim3(tokens), dim3(256), 0, stream, (const bf16_t*)x,
+                           (bf16_t*)out, cols, coef, eps);
     else if (act_type == RL_BF16)
-        hipLaunchKernelGGL(polynorm_kernel<bf16_t>, dim3(tokens), dim3(256), 0, stream, (const bf16_t*)x,
+        hipLaunchKernelGGL((polynorm_kernel<bf16_t, 1>), dim3(tokens), dim3(256), 0, stream, (const bf16_t*)x,
                            (bf16_t*)out, cols, coef, eps);
     else
         return RL_ERR_ARG;

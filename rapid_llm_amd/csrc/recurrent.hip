@@ -6,9 +6,19 @@
 //
 // A step is a flat batch of requests: request s brings the tokens cu[s] .. cu[s + 1] - 1 and keeps
 // its state in row seq_slots[s] of the state tensors.  Every scan walks a request's tokens in
-// order with the state in registers, one workgroup per (request, head), so a token's sums are
-// formed in one order whatever else the step holds and however the request's tokens were cut into
-// steps: in float32 the results are equal bit for bit.
+// order with the state in registers, so a token's sums are formed in one order whatever else the
+// step holds and however the request's tokens were cut into steps: in float32 the results are
+// equal bit for bit.
+//
+// How a scan is laid out.  A head's state is a matrix [rows i, columns j]; a token multiplies
+// every element once or twice and sums over the rows, and the next token cannot start before.
+// What bounds a prompt is therefore the time of one token, and that is the state elements a lane
+// holds: a wave takes 4 columns and deals the rows to its 16 lanes a column (RPL rows a lane),
+// a workgroup of 4 waves takes 16 columns, a head is ceil(columns / 16) workgroups on compute
+// units of their own.  The row sums are folded over the 16 lanes by four rotations inside the
+// row of lanes (data-parallel primitives, no trip through LDS).  The tokens' operands come
+// through LDS sixteen tokens at a time, the next sixteen travelling from memory meanwhile.  The
+// state is kept column-major ([j][i]) so that a lane's rows are contiguous.
 #include "common.h"
 
 namespace recurrent {
@@ -32,29 +42,75 @@ __device__ inline float silu(float z) { return z / (1.f + expf(-z)); }
 // Token shift.  With h' the previous token's row (the request's state row before its first token
 // of the step), branch b reads h + (h' - h) * mu[b].  Branches 0..3 are written in the compute
 // type, side by side as [4][tokens][width]; branch 4 (the decay's) in float32.
-// The state row is replaced by the request's last row in a second launch, after every read.
+// The state row is replaced by the request's last row in a second launch, after every read; in a
+// step of single tokens (`single`) a token's workgroup is the only one that touches its request's
+// row and replaces it itself.
 // --------------------------------------------------------------------------- //
 template <typename T>
+struct alignas(sizeof(T) * 4) Quad {
+    T v[4];
+};
+
+template <typename T>
 __global__ __launch_bounds__(256) void token_shift_kernel(const T* __restrict__ x, const float* __restrict__ mu,
-                                                          const float* __restrict__ state, T* __restrict__ mixes,
+                                                          float* __restrict__ state, T* __restrict__ mixes,
                                                           float* __restrict__ mix_w, const int* __restrict__ cu,
                                                           const int* __restrict__ seq_slots, int num_seqs,
-                                                          int tokens, int width) {
+                                                          int tokens, int width, int single) {
     const int t = blockIdx.x;
-    const int s = request_of(cu, num_seqs, t);
-    const bool first = t == cu[s];
-    const float* prev_state = state + (size_t)seq_slots[s] * width;
+    const int s = single ? t : request_of(cu, num_seqs, t);
+    const bool first = single || t == cu[s];
+    float* prev_state = state + (size_t)seq_slots[s] * width;
     const T* row = x + (size_t)t * width;
     const T* before = x + (size_t)(first ? t : t - 1) * width;
     const size_t plane = (size_t)tokens * width;
+    if (width % 4 == 0) {
+        // four channels a thread, every access 8 or 16 bytes; the loads of two rounds are asked for together
+#pragma unroll 2
+        for (int i = 4 * threadIdx.x; i < width; i += 4 * blockDim.x) {
+            const Quad<T> hq = *reinterpret_cast<const Quad<T>*>(row + i);
+            float p[4];
+            if (first) {
+                const float4 ps = *reinterpret_cast<const float4*>(prev_state + i);
+                p[0] = ps.x; p[1] = ps.y; p[2] = ps.z; p[3] = ps.w;
+            } else {
+                const Quad<T> pq = *reinterpret_cast<const Quad<T>*>(before + i);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) p[e] = to_float(pq.v[e]);
+            }
+            float h[4], d[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                h[e] = to_float(hq.v[e]);
+                d[e] = p[e] - h[e];
+            }
+#pragma unroll
+            for (int b = 0; b < 5; ++b) {
+                const float4 m = *reinterpret_cast<const float4*>(mu + (size_t)b * width + i);
+                const float y[4] = {fmaf(d[0], m.x, h[0]), fmaf(d[1], m.y, h[1]), fmaf(d[2], m.z, h[2]),
+                                    fmaf(d[3], m.w, h[3])};
+                if (b < 4) {
+                    Quad<T> o;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o.v[e] = from_float<T>(y[e]);
+                    *reinterpret_cast<Quad<T>*>(mixes + b * plane + (size_t)t * width + i) = o;
+                } else {
+                    *reinterpret_cast<float4*>(mix_w + (size_t)t * width + i) = make_float4(y[0], y[1], y[2], y[3]);
+                }
+            }
+            if (single) *reinterpret_cast<float4*>(prev_state + i) = make_float4(h[0], h[1], h[2], h[3]);
+        }
+        return;
+    }
     for (int i = threadIdx.x; i < width; i += blockDim.x) {
         const float h = to_float(row[i]);
         const float p = first ? prev_state[i] : to_float(before[i]);
         const float d = p - h;
 #pragma unroll
         for (int b = 0; b < 4; ++b)
-            mixes[b * plane + (size_t)t * width + i] = from_float<T>(h + d * mu[(size_t)b * width + i]);
-        mix_w[(size_t)t * width + i] = h + d * mu[(size_t)4 * width + i];
+            mixes[b * plane + (size_t)t * width + i] = from_float<T>(fmaf(d, mu[(size_t)b * width + i], h));
+        mix_w[(size_t)t * width + i] = fmaf(d, mu[(size_t)4 * width + i], h);
+        if (single) prev_state[i] = h;
     }
 }
 
@@ -69,99 +125,194 @@ __global__ __launch_bounds__(256) void shift_state_kernel(const T* __restrict__ 
 }
 
 // --------------------------------------------------------------------------- //
-// The time-mixing scan.  Per head, state S[key channel i][value channel j]; thread j keeps column
-// j in registers.  For a token with r, k, v (d each), decay w_i = exp(-exp(pre_i + bias_i)) and
-// the bonus u_i:
-//   o_j = sum_i r_i (S_ij + u_i k_i v_j)        S_ij <- w_i S_ij + k_i v_j
-// then o is divided by its root mean square over the head, multiplied by the norm's weight and by
-// silu(g).  The next token's operands travel while this one is computed.
+// Helpers of the scans: the sum over a row of 16 lanes by rotations (every lane gets it; the
+// order of the additions is fixed by the lane), and the block of tokens staged in LDS.
 // --------------------------------------------------------------------------- //
-template <typename T, int DMAX>
-__global__ __launch_bounds__(DMAX < 64 ? 64 : DMAX) void wkv_scan_kernel(
-    const T* __restrict__ r, const T* __restrict__ k, const T* __restrict__ v, const T* __restrict__ g,
-    const float* __restrict__ decay_pre, const float* __restrict__ decay_bias, const float* __restrict__ bonus,
-    const float* __restrict__ norm_w, T* __restrict__ out, const int* __restrict__ cu,
-    const int* __restrict__ seq_slots, float* __restrict__ S, int heads, int d, float eps) {
-    const int s = blockIdx.x, h = blockIdx.y, j = threadIdx.x;
+template <int CTRL>
+__device__ inline float ror_add(float v) {
+    const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false);
+    return v + __int_as_float(moved);
+}
+__device__ inline float row16_sum(float v) {
+    v = ror_add<0x128>(v);  // row_ror:8
+    v = ror_add<0x124>(v);  // row_ror:4
+    v = ror_add<0x122>(v);  // row_ror:2
+    v = ror_add<0x121>(v);  // row_ror:1
+    return v;
+}
+
+constexpr int SCAN_TOKENS = 16;   // tokens staged at a time
+constexpr int SCAN_THREADS = 256;  // 4 waves: 16 columns
+
+// --------------------------------------------------------------------------- //
+// The time-mixing scan.  Per head, state S[key channel i][value channel j], kept as [j][i].  For a
+// token with r, k, v (d each), the decay w_i = exp(-exp(pre_i + bias_i)), formed as a block of
+// tokens is fetched, and the bonus u_i:
+//   o_j = sum_i r_i (S_ij + u_i k_i v_j)        S_ij <- w_i S_ij + k_i v_j
+// o goes out unfinished (float32); wkv_finish_kernel divides every head by its root mean square
+// and applies the norm's weight and silu(g).
+// --------------------------------------------------------------------------- //
+// one state element's share of a token (the same instructions wherever a token is computed)
+__device__ inline void wkv_row(float r, float k, float w, float u, float vj, float& state, float& o) {
+    const float kv = k * vj;
+    o = fmaf(r, fmaf(u, kv, state), o);
+    state = fmaf(w, state, kv);
+}
+__device__ inline float wkv_decay(float pre, float bias) { return expf(-expf(pre + bias)); }
+
+template <typename T, int RPL>
+__global__ __launch_bounds__(SCAN_THREADS) void wkv_scan_kernel(
+    const T* __restrict__ r, const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ decay_pre,
+    const float* __restrict__ decay_bias, const float* __restrict__ bonus, float* __restrict__ raw,
+    const int* __restrict__ cu,
+    const int* __restrict__ seq_slots, float* __restrict__ S, int heads, int d) {
+    constexpr int DP = 16 * RPL;  // rows, padded
+    constexpr int PER_THREAD = SCAN_TOKENS * DP / SCAN_THREADS;  // = RPL
+    const int s = blockIdx.x, h = blockIdx.y;
     const int t0 = cu[s], t1 = cu[s + 1];
     const int inner = heads * d;
+    const int lane = threadIdx.x & (RL_WAVE - 1), wave = threadIdx.x / RL_WAVE;
+    const int c = lane & 15;                                  // which share of the rows
+    const int col = wave * 4 + (lane >> 4);                   // column of the workgroup's 16
+    const int j = blockIdx.z * 16 + col;
     const bool live = j < d;
-    const int col = h * d + (live ? j : 0);
-    __shared__ float sr[DMAX], sk[DMAX], sw[DMAX], su[DMAX];
-    __shared__ float scratch[16];
-    float* Sp = S + ((size_t)seq_slots[s] * heads + h) * d * d;
-    float state[DMAX];
+    __shared__ __attribute__((aligned(16))) float sr[SCAN_TOKENS][DP], sk[SCAN_TOKENS][DP], sw[SCAN_TOKENS][DP];
+    __shared__ float sv[SCAN_TOKENS][16];
+    float* Sp = S + (((size_t)seq_slots[s] * heads + h) * d + (live ? j : 0)) * d;
+    float state[RPL], u[RPL];
 #pragma unroll
-    for (int i = 0; i < DMAX; ++i) state[i] = (live && i < d) ? Sp[(size_t)i * d + j] : 0.f;
-    const float bias = decay_bias[col], nw = norm_w[col];
-    if (live) su[j] = bonus[col];
-    float nr = 0.f, nk = 0.f, nv = 0.f, ng = 0.f, np = 0.f;
-    if (t0 < t1) {
-        const size_t at = (size_t)t0 * inner + col;
-        nr = to_float(r[at]); nk = to_float(k[at]); nv = to_float(v[at]); ng = to_float(g[at]); np = decay_pre[at];
+    for (int ii = 0; ii < RPL; ++ii) {
+        const int i = c * RPL + ii;
+        state[ii] = (live && i < d) ? Sp[i] : 0.f;
+        u[ii] = i < d ? bonus[h * d + i] : 0.f;
     }
-    for (int t = t0; t < t1; ++t) {
-        __syncthreads();  // the token before has been read by every thread
-        if (live) {
-            sr[j] = nr;
-            sk[j] = nk;
-            sw[j] = expf(-expf(np + bias));
-        }
-        const float vj = live ? nv : 0.f, gj = ng;
-        __syncthreads();
-        if (t + 1 < t1) {
-            const size_t at = (size_t)(t + 1) * inner + col;
-            nr = to_float(r[at]); nk = to_float(k[at]); nv = to_float(v[at]); ng = to_float(g[at]); np = decay_pre[at];
-        }
-        float o = 0.f;
+    // a block of tokens from memory into registers: element e of the block's [token][row] arrays
+    float pr[PER_THREAD], pk[PER_THREAD], pw[PER_THREAD], pv = 0.f;
+    auto fetch = [&](int tb) {
 #pragma unroll
-        for (int i = 0; i < DMAX; ++i) {
-            if (i < d) {
-                const float kv = sk[i] * vj;
-                o += sr[i] * (state[i] + su[i] * kv);
-                state[i] = sw[i] * state[i] + kv;
-            }
+        for (int e = 0; e < PER_THREAD; ++e) {
+            const int idx = e * SCAN_THREADS + threadIdx.x;
+            const int tt = idx / DP, i = idx % DP;
+            const bool ok = tb + tt < t1 && i < d;
+            const size_t at = (size_t)(tb + tt) * inner + h * d + i;
+            pr[e] = ok ? to_float(r[at]) : 0.f;
+            pk[e] = ok ? to_float(k[at]) : 0.f;
+            pw[e] = ok ? wkv_decay(decay_pre[at], decay_bias[h * d + i]) : 0.f;
         }
-        const float ss = block_sum(live ? o * o : 0.f, scratch);
-        const float rr = rsqrtf(ss / (float)d + eps);
-        if (live) out[(size_t)t * inner + col] = from_float<T>(o * rr * nw * silu(gj));
+        const int tt = threadIdx.x / 16, jj = blockIdx.z * 16 + (threadIdx.x & 15);
+        pv = (tb + tt < t1 && jj < d) ? to_float(v[(size_t)(tb + tt) * inner + h * d + jj]) : 0.f;
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int e = 0; e < PER_THREAD; ++e) {
+            const int idx = e * SCAN_THREADS + threadIdx.x;
+            (&sr[0][0])[idx] = pr[e];
+            (&sk[0][0])[idx] = pk[e];
+            (&sw[0][0])[idx] = pw[e];
+        }
+        (&sv[0][0])[threadIdx.x] = pv;
+    };
+    fetch(t0);
+    for (int tb = t0; tb < t1; tb += SCAN_TOKENS) {
+        __syncthreads();  // the block before has been read by every wave
+        stage();
+        __syncthreads();
+        if (tb + SCAN_TOKENS < t1) fetch(tb + SCAN_TOKENS);
+        const int nt = min(SCAN_TOKENS, t1 - tb);
+        auto token = [&](int tt) {
+            const float vj = sv[tt][col];
+            float o = 0.f;
+#pragma unroll
+            for (int ii = 0; ii < RPL; ++ii)
+                wkv_row(sr[tt][c * RPL + ii], sk[tt][c * RPL + ii], sw[tt][c * RPL + ii], u[ii], vj, state[ii], o);
+            o = row16_sum(o);
+            if (c == 0 && live) raw[(size_t)(tb + tt) * inner + h * d + j] = o;
+        };
+        if (nt == SCAN_TOKENS) {
+            // a whole block, unrolled: the reads of later tokens stand in front of the sums of
+            // earlier ones, and only the state's own chain orders the tokens
+#pragma unroll
+            for (int tt = 0; tt < SCAN_TOKENS; ++tt) token(tt);
+        } else {
+            for (int tt = 0; tt < nt; ++tt) token(tt);
+        }
     }
     if (live) {
 #pragma unroll
-        for (int i = 0; i < DMAX; ++i)
-            if (i < d) Sp[(size_t)i * d + j] = state[i];
+        for (int ii = 0; ii < RPL; ++ii)
+            if (c * RPL + ii < d) Sp[c * RPL + ii] = state[ii];
     }
+}
+
+// out[t, head] = raw / sqrt(mean(raw^2) + eps) * norm_w * silu(g): one wave a (token, head)
+template <typename T>
+__global__ __launch_bounds__(256) void wkv_finish_kernel(const float* __restrict__ raw, const T* __restrict__ g,
+                                                         const float* __restrict__ norm_w, T* __restrict__ out,
+                                                         int rows, int heads, int d, float eps) {
+    const int row = blockIdx.x * 4 + threadIdx.x / RL_WAVE;  // (token, head)
+    const int lane = threadIdx.x & (RL_WAVE - 1);
+    if (row >= rows) return;  // whole waves leave
+    const size_t base = (size_t)row * d;
+    const int h = row % heads;
+    float ss = 0.f;
+    for (int i = lane; i < d; i += RL_WAVE) {
+        const float o = raw[base + i];
+        ss += o * o;
+    }
+    const float rr = rsqrtf(wave_sum(ss) / (float)d + eps);
+    for (int i = lane; i < d; i += RL_WAVE)
+        out[base + i] = from_float<T>(raw[base + i] * rr * norm_w[h * d + i] * silu(to_float(g[base + i])));
 }
 
 // --------------------------------------------------------------------------- //
 // Causal convolution per channel over the columns [col0, col0 + channels) of the packed rows, with
 // bias and silu: y_t = silu(b + sum_tap w[c][tap] in(t - (taps - 1) + tap)), where inputs before
 // the request's first token of the step come from its state rows (the last taps - 1 inputs it has
-// seen, oldest first; zeros when the request begins).  A second launch then shifts the state.
+// seen, oldest first; zeros when the request begins).  A second launch then shifts the state; in a
+// step of single tokens (`single`) the thread of a channel shifts its request's rows itself.
 // --------------------------------------------------------------------------- //
 #define RL_CONV_MAX_TAPS 8
+
+constexpr int CONV_TOKENS = 8;  // consecutive tokens of the flat batch a workgroup takes in a step with portions
 
 template <typename T>
 __global__ __launch_bounds__(256) void causal_conv_kernel(const T* __restrict__ packed, int row_width, int col0,
                                                           const float* __restrict__ w, const float* __restrict__ bias,
-                                                          const float* __restrict__ state, float* __restrict__ out,
+                                                          float* __restrict__ state, float* __restrict__ out,
                                                           const int* __restrict__ cu,
-                                                          const int* __restrict__ seq_slots, int num_seqs,
-                                                          int channels, int taps) {
-    const int t = blockIdx.x;
-    const int s = request_of(cu, num_seqs, t);
-    const int offset = t - cu[s];  // tokens of the request's portion before this one
+                                                          const int* __restrict__ seq_slots, int num_seqs, int tokens,
+                                                          int channels, int taps, int single, int per_group) {
+    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (c >= channels) return;
     const int held = taps - 1;
-    const float* st = state + (size_t)seq_slots[s] * max(held, 1) * channels;
-    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < channels; c += gridDim.y * blockDim.x) {
-        float acc = bias[c];
-        for (int tap = 0; tap < taps; ++tap) {
-            const int rel = offset - held + tap;  // offset in the portion of the input this tap meets
-            const float in = rel >= 0 ? to_float(packed[(size_t)(t - offset + rel) * row_width + col0 + c])
-                                      : st[(size_t)(held + rel) * channels + c];
-            acc = fmaf(w[(size_t)c * taps + tap], in, acc);
+    float wt[RL_CONV_MAX_TAPS];  // this channel's taps
+#pragma unroll
+    for (int tap = 0; tap < RL_CONV_MAX_TAPS; ++tap) wt[tap] = tap < taps ? w[(size_t)c * taps + tap] : 0.f;
+    const float b = bias[c];
+    const int first = blockIdx.x * per_group;
+    int s = single ? first : request_of(cu, num_seqs, first);
+    for (int t = first; t < min(tokens, first + per_group); ++t) {
+        if (single)
+            s = t;
+        else
+            while (t >= cu[s + 1]) ++s;  // tokens ascend through the requests
+        const int offset = single ? 0 : t - cu[s];  // tokens of the request's portion before this one
+        float* st = state + (size_t)seq_slots[s] * max(held, 1) * channels;
+        float acc = b;
+#pragma unroll
+        for (int tap = 0; tap < RL_CONV_MAX_TAPS; ++tap) {
+            if (tap < taps) {
+                const int rel = offset - held + tap;  // offset in the portion of the input this tap meets
+                const float in = rel >= 0 ? to_float(packed[(size_t)(t - offset + rel) * row_width + col0 + c])
+                                          : st[(size_t)(held + rel) * channels + c];
+                acc = fmaf(wt[tap], in, acc);
+            }
         }
         out[(size_t)t * channels + c] = silu(acc);
+        if (single && held > 0) {
+            for (int q = 0; q + 1 < held; ++q) st[(size_t)q * channels + c] = st[(size_t)(q + 1) * channels + c];
+            st[(size_t)(held - 1) * channels + c] = to_float(packed[(size_t)t * row_width + col0 + c]);
+        }
     }
 }
 
@@ -196,73 +347,110 @@ __global__ __launch_bounds__(256) void conv_state_kernel(const T* __restrict__ p
 
 // --------------------------------------------------------------------------- //
 // The state-space scan.  `mixed` rows are [x: heads * P | B: groups * N | C: groups * N] (float32,
-// behind convolution and silu); per head, state S[n][p], thread p keeps column p in registers:
-//   dt = softplus(dt_raw + dt_bias)     a = exp(-exp(A_log) dt)
+// behind convolution and silu); per head, state S[n][p], kept as [p][n].  As a block of tokens is
+// fetched the raw step sizes become dt = softplus(dt_raw + dt_bias) and a = exp(-exp(A_log) dt); then
 //   S_np <- a S_np + dt B_n x_p          y_p = sum_n S_np C_n + D x_p
 // and y_p silu(z_p) is written (z: the first heads * P columns of the packed rows).
 // --------------------------------------------------------------------------- //
-template <typename T, int NMAX>
-__global__ __launch_bounds__(256) void ssm_scan_kernel(
+__device__ inline float ssm_step_size(float raw, float bias) {
+    const float pre = raw + bias;
+    return pre > 20.f ? pre : log1pf(expf(pre));
+}
+__device__ inline float ssm_decay(float a_log, float dt) { return expf(-expf(a_log) * dt); }
+// one state element's share of a token, and the finished output of a channel
+__device__ inline void ssm_row(float a, float B, float C, float dx, float& state, float& y) {
+    state = fmaf(B, dx, a * state);
+    y = fmaf(state, C, y);
+}
+__device__ inline float ssm_out(float y, float D, float x, float z) { return fmaf(D, x, y) * silu(z); }
+
+template <typename T, int RPL>
+__global__ __launch_bounds__(SCAN_THREADS) void ssm_scan_kernel(
     const float* __restrict__ mixed, const float* __restrict__ dt_raw, const float* __restrict__ dt_bias,
-    const float* __restrict__ a_log, const float* __restrict__ skip, const T* __restrict__ packed, int row_width,
-    float* __restrict__ out, const int* __restrict__ cu, const int* __restrict__ seq_slots,
-    float* __restrict__ S, int heads, int P, int N, int groups) {
-    const int s = blockIdx.x, h = blockIdx.y, p = threadIdx.x;
+    const float* __restrict__ a_log, const float* __restrict__ skip, const T* __restrict__ packed, int row_width, float* __restrict__ out, const int* __restrict__ cu,
+    const int* __restrict__ seq_slots, float* __restrict__ S, int heads, int P, int N, int groups) {
+    constexpr int NP = 16 * RPL;  // state rows, padded
+    constexpr int PER_THREAD = SCAN_TOKENS * NP / SCAN_THREADS;  // = RPL
+    const int s = blockIdx.x, h = blockIdx.y;
     const int t0 = cu[s], t1 = cu[s + 1];
     const int inner = heads * P;
     const int channels = inner + 2 * groups * N;
     const int grp = h / (heads / groups);
+    const int lane = threadIdx.x & (RL_WAVE - 1), wave = threadIdx.x / RL_WAVE;
+    const int c = lane & 15;
+    const int col = wave * 4 + (lane >> 4);
+    const int p = blockIdx.z * 16 + col;
     const bool live = p < P;
-    const bool feeds = p < N;  // this thread also carries B_n and C_n of n = p into LDS
-    __shared__ float sB[NMAX], sC[NMAX];
-    float* Sp = S + ((size_t)seq_slots[s] * heads + h) * N * P;
-    float state[NMAX];
+    __shared__ __attribute__((aligned(16))) float sB[SCAN_TOKENS][NP], sC[SCAN_TOKENS][NP];
+    __shared__ float sx[SCAN_TOKENS][16], sz[SCAN_TOKENS][16], sdt[SCAN_TOKENS], sa[SCAN_TOKENS];
+    float* Sp = S + (((size_t)seq_slots[s] * heads + h) * P + (live ? p : 0)) * N;
+    float state[RPL];
 #pragma unroll
-    for (int n = 0; n < NMAX; ++n) state[n] = (live && n < N) ? Sp[(size_t)n * P + p] : 0.f;
-    const float bias = dt_bias[h], rate = expf(a_log[h]), D = skip[h];
-    const int xcol = h * P + (live ? p : 0);
-    const int bcol = inner + grp * N + (feeds ? p : 0);
-    const int ccol = bcol + groups * N;
-    float nx = 0.f, nb = 0.f, nc = 0.f, nz = 0.f, nd = 0.f;
-    if (t0 < t1) {
-        const float* row = mixed + (size_t)t0 * channels;
-        nx = row[xcol]; nb = row[bcol]; nc = row[ccol];
-        nz = to_float(packed[(size_t)t0 * row_width + xcol]);
-        nd = dt_raw[(size_t)t0 * heads + h];
-    }
-    for (int t = t0; t < t1; ++t) {
-        __syncthreads();  // the token before has been read by every thread
-        if (feeds) {
-            sB[p] = nb;
-            sC[p] = nc;
+    for (int ii = 0; ii < RPL; ++ii) state[ii] = (live && c * RPL + ii < N) ? Sp[c * RPL + ii] : 0.f;
+    const float D = skip[h];
+    float pB[PER_THREAD], pC[PER_THREAD], px = 0.f, pz = 0.f, pd = 0.f;
+    auto fetch = [&](int tb) {
+#pragma unroll
+        for (int e = 0; e < PER_THREAD; ++e) {
+            const int idx = e * SCAN_THREADS + threadIdx.x;
+            const int tt = idx / NP, n = idx % NP;
+            const bool ok = tb + tt < t1 && n < N;
+            const float* row = mixed + (size_t)(tb + tt) * channels + inner + grp * N + n;
+            pB[e] = ok ? row[0] : 0.f;
+            pC[e] = ok ? row[groups * N] : 0.f;
         }
-        const float x = live ? nx : 0.f, z = nz;
-        const float pre = nd + bias;
-        const float dt = pre > 20.f ? pre : log1pf(expf(pre));
-        const float a = expf(-rate * dt);
+        const int tt = threadIdx.x / 16, pp = blockIdx.z * 16 + (threadIdx.x & 15);
+        const bool ok = tb + tt < t1 && pp < P;
+        px = ok ? mixed[(size_t)(tb + tt) * channels + h * P + pp] : 0.f;
+        pz = ok ? to_float(packed[(size_t)(tb + tt) * row_width + h * P + pp]) : 0.f;
+        // threads 0..15 carry the step sizes, threads 16..31 the decays of the block's tokens
+        const int which = threadIdx.x / 16, tk = threadIdx.x & 15;
+        pd = 0.f;
+        if (which < 2 && tb + tk < t1) {
+            const float dt = ssm_step_size(dt_raw[(size_t)(tb + tk) * heads + h], dt_bias[h]);
+            pd = which == 0 ? dt : ssm_decay(a_log[h], dt);
+        }
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int e = 0; e < PER_THREAD; ++e) {
+            const int idx = e * SCAN_THREADS + threadIdx.x;
+            (&sB[0][0])[idx] = pB[e];
+            (&sC[0][0])[idx] = pC[e];
+        }
+        (&sx[0][0])[threadIdx.x] = px;
+        (&sz[0][0])[threadIdx.x] = pz;
+        if (threadIdx.x < 16) sdt[threadIdx.x] = pd;
+        else if (threadIdx.x < 32) sa[threadIdx.x - 16] = pd;
+    };
+    fetch(t0);
+    for (int tb = t0; tb < t1; tb += SCAN_TOKENS) {
+        __syncthreads();  // the block before has been read by every wave
+        stage();
         __syncthreads();
-        if (t + 1 < t1) {
-            const float* row = mixed + (size_t)(t + 1) * channels;
-            nx = row[xcol]; nb = row[bcol]; nc = row[ccol];
-            nz = to_float(packed[(size_t)(t + 1) * row_width + xcol]);
-            nd = dt_raw[(size_t)(t + 1) * heads + h];
-        }
-        const float dx = dt * x;
-        float y = 0.f;
+        if (tb + SCAN_TOKENS < t1) fetch(tb + SCAN_TOKENS);
+        const int nt = min(SCAN_TOKENS, t1 - tb);
+        auto token = [&](int tt) {
+            const float x = sx[tt][col], a = sa[tt];
+            const float dx = sdt[tt] * x;
+            float y = 0.f;
 #pragma unroll
-        for (int n = 0; n < NMAX; ++n) {
-            if (n < N) {
-                state[n] = a * state[n] + sB[n] * dx;
-                y += state[n] * sC[n];
-            }
+            for (int ii = 0; ii < RPL; ++ii)
+                ssm_row(a, sB[tt][c * RPL + ii], sC[tt][c * RPL + ii], dx, state[ii], y);
+            y = row16_sum(y);
+            if (c == 0 && live) out[(size_t)(tb + tt) * inner + h * P + p] = ssm_out(y, D, x, sz[tt][col]);
+        };
+        if (nt == SCAN_TOKENS) {
+#pragma unroll
+            for (int tt = 0; tt < SCAN_TOKENS; ++tt) token(tt);
+        } else {
+            for (int tt = 0; tt < nt; ++tt) token(tt);
         }
-        y += D * x;
-        if (live) out[(size_t)t * inner + xcol] = y * silu(z);
     }
     if (live) {
 #pragma unroll
-        for (int n = 0; n < NMAX; ++n)
-            if (n < N) Sp[(size_t)n * P + p] = state[n];
+        for (int ii = 0; ii < RPL; ++ii)
+            if (c * RPL + ii < N) Sp[c * RPL + ii] = state[ii];
     }
 }
 
@@ -294,16 +482,19 @@ extern "C" int rl_token_shift(const void* x, const float* mu, float* state, void
                               int act_type, hipStream_t stream) {
     if (tokens <= 0 || num_seqs <= 0) return RL_OK;
     if (width < 1) return RL_ERR_ARG;
+    const int single = tokens == num_seqs;  // every request brings one token
     if (act_type == RL_F32) {
         hipLaunchKernelGGL(recurrent::token_shift_kernel<float>, dim3(tokens), dim3(256), 0, stream, (const float*)x,
-                           mu, state, (float*)mixes, mix_w, cu, seq_slots, num_seqs, tokens, width);
-        hipLaunchKernelGGL(recurrent::shift_state_kernel<float>, dim3(num_seqs), dim3(256), 0, stream,
+                           mu, state, (float*)mixes, mix_w, cu, seq_slots, num_seqs, tokens, width, single);
+        if (!single)
+            hipLaunchKernelGGL(recurrent::shift_state_kernel<float>, dim3(num_seqs), dim3(256), 0, stream,
                            (const float*)x, state, cu, seq_slots, width);
     } else if (act_type == RL_BF16) {
         hipLaunchKernelGGL(recurrent::token_shift_kernel<bf16_t>, dim3(tokens), dim3(256), 0, stream,
                            (const bf16_t*)x, mu, state, (bf16_t*)mixes, mix_w, cu, seq_slots, num_seqs, tokens,
-                           width);
-        hipLaunchKernelGGL(recurrent::shift_state_kernel<bf16_t>, dim3(num_seqs), dim3(256), 0, stream,
+                           width, single);
+        if (!single)
+            hipLaunchKernelGGL(recurrent::shift_state_kernel<bf16_t>, dim3(num_seqs), dim3(256), 0, stream,
                            (const bf16_t*)x, state, cu, seq_slots, width);
     } else {
         return RL_ERR_ARG;
@@ -312,40 +503,48 @@ extern "C" int rl_token_shift(const void* x, const float* mu, float* state, void
 }
 
 template <typename T>
-static int launch_wkv(const T* r, const T* k, const T* v, const T* g, const float* decay_pre,
-                      const float* decay_bias, const float* bonus, const float* norm_w, T* out, const int* cu,
-                      const int* seq_slots, float* S, int num_seqs, int heads, int d, float eps,
+static int launch_wkv(const T* r, const T* k, const T* v, const T* g, const float* decay, const float* decay_bias,
+                      const float* bonus, const float* norm_w, T* out, float* raw, const int* cu,
+                      const int* seq_slots, float* S, int num_seqs, int tokens, int heads, int d, float eps,
                       hipStream_t stream) {
-    dim3 grid(num_seqs, heads);
-#define RL_WKV(DMAX)                                                                                            \
-    hipLaunchKernelGGL((recurrent::wkv_scan_kernel<T, DMAX>), grid, dim3(DMAX < 64 ? 64 : DMAX), 0, stream, r, k, v, \
-                       g, decay_pre, decay_bias, bonus, norm_w, out, cu, seq_slots, S, heads, d, eps)
-    if (d <= 32)
-        RL_WKV(32);
-    else if (d <= 64)
-        RL_WKV(64);
-    else if (d <= 128)
-        RL_WKV(128);
+    dim3 grid(num_seqs, heads, (d + 15) / 16);
+#define RL_WKV(RPL)                                                                                              \
+    hipLaunchKernelGGL((recurrent::wkv_scan_kernel<T, RPL>), grid, dim3(recurrent::SCAN_THREADS), 0, stream, r, k, v, \
+                       decay, decay_bias, bonus, raw, cu, seq_slots, S, heads, d)
+    const int rows = (d + 15) / 16;
+    if (rows <= 1)
+        RL_WKV(1);
+    else if (rows <= 2)
+        RL_WKV(2);
+    else if (rows <= 4)
+        RL_WKV(4);
+    else if (rows <= 8)
+        RL_WKV(8);
     else
-        RL_WKV(256);
+        RL_WKV(16);
 #undef RL_WKV
+    const int heads_rows = tokens * heads;
+    hipLaunchKernelGGL(recurrent::wkv_finish_kernel<T>, dim3((heads_rows + 3) / 4), dim3(256), 0, stream, raw, g,
+                       norm_w, out, heads_rows, heads, d, eps);
     return rl_launch_status();
 }
 
-extern "C" int rl_wkv_scan(const void* r, const void* k, const void* v, const void* g, const float* decay_pre,
+// decay: the decays' pre-activations [tokens, heads * d]; raw: [tokens, heads * d] float32 scratch
+// for the unfinished outputs
+extern "C" int rl_wkv_scan(const void* r, const void* k, const void* v, const void* g, const float* decay,
                            const float* decay_bias, const float* bonus, const float* norm_w, void* out,
-                           const int* cu, const int* seq_slots, float* S, int num_seqs, int heads, int d,
-                           float eps, int act_type, hipStream_t stream) {
-    if (num_seqs <= 0) return RL_OK;
-    if (heads < 1 || heads > 65535 || d < 1 || d > 256) return RL_ERR_ARG;
+                           float* raw, const int* cu, const int* seq_slots, float* S, int num_seqs, int tokens,
+                           int heads, int d, float eps, int act_type, hipStream_t stream) {
+    if (num_seqs <= 0 || tokens <= 0) return RL_OK;
+    if (heads < 1 || heads > 65535 || d < 1 || d > 256 || num_seqs > 65535) return RL_ERR_ARG;
     if (act_type == RL_F32)
-        return launch_wkv<float>((const float*)r, (const float*)k, (const float*)v, (const float*)g, decay_pre,
-                                 decay_bias, bonus, norm_w, (float*)out, cu, seq_slots, S, num_seqs, heads, d, eps,
-                                 stream);
+        return launch_wkv<float>((const float*)r, (const float*)k, (const float*)v, (const float*)g, decay,
+                                 decay_bias, bonus, norm_w, (float*)out, raw, cu, seq_slots, S, num_seqs, tokens,
+                                 heads, d, eps, stream);
     if (act_type == RL_BF16)
-        return launch_wkv<bf16_t>((const bf16_t*)r, (const bf16_t*)k, (const bf16_t*)v, (const bf16_t*)g, decay_pre,
-                                  decay_bias, bonus, norm_w, (bf16_t*)out, cu, seq_slots, S, num_seqs, heads, d,
-                                  eps, stream);
+        return launch_wkv<bf16_t>((const bf16_t*)r, (const bf16_t*)k, (const bf16_t*)v, (const bf16_t*)g, decay,
+                                  decay_bias, bonus, norm_w, (bf16_t*)out, raw, cu, seq_slots, S, num_seqs, tokens,
+                                  heads, d, eps, stream);
     return RL_ERR_ARG;
 }
 
@@ -356,17 +555,21 @@ extern "C" int rl_causal_conv(const void* packed, int row_width, int col0, const
     if (channels < 1 || taps < 1 || taps > RL_CONV_MAX_TAPS || col0 < 0 || col0 + channels > row_width)
         return RL_ERR_ARG;
     const int cblocks = (channels + 255) / 256;
-    dim3 grid(tokens, cblocks > 64 ? 64 : cblocks), sgrid(num_seqs, cblocks);
+    const int single = tokens == num_seqs;  // every request brings one token
+    if (cblocks > 65535) return RL_ERR_ARG;
+    // single tokens: a workgroup a token, so that no token waits for another
+    const int per_group = single ? 1 : recurrent::CONV_TOKENS;
+    dim3 grid((tokens + per_group - 1) / per_group, cblocks), sgrid(num_seqs, cblocks);
     if (act_type == RL_F32) {
         hipLaunchKernelGGL(recurrent::causal_conv_kernel<float>, grid, dim3(256), 0, stream, (const float*)packed,
-                           row_width, col0, w, bias, state, out, cu, seq_slots, num_seqs, channels, taps);
-        if (taps > 1)
+                           row_width, col0, w, bias, state, out, cu, seq_slots, num_seqs, tokens, channels, taps, single, per_group);
+        if (taps > 1 && !single)
             hipLaunchKernelGGL(recurrent::conv_state_kernel<float>, sgrid, dim3(256), 0, stream,
                                (const float*)packed, row_width, col0, state, cu, seq_slots, channels, taps);
     } else if (act_type == RL_BF16) {
         hipLaunchKernelGGL(recurrent::causal_conv_kernel<bf16_t>, grid, dim3(256), 0, stream, (const bf16_t*)packed,
-                           row_width, col0, w, bias, state, out, cu, seq_slots, num_seqs, channels, taps);
-        if (taps > 1)
+                           row_width, col0, w, bias, state, out, cu, seq_slots, num_seqs, tokens, channels, taps, single, per_group);
+        if (taps > 1 && !single)
             hipLaunchKernelGGL(recurrent::conv_state_kernel<bf16_t>, sgrid, dim3(256), 0, stream,
                                (const bf16_t*)packed, row_width, col0, state, cu, seq_slots, channels, taps);
     } else {
@@ -378,42 +581,41 @@ extern "C" int rl_causal_conv(const void* packed, int row_width, int col0, const
 template <typename T>
 static int launch_ssm(const float* mixed, const float* dt_raw, const float* dt_bias, const float* a_log,
                       const float* skip, const T* packed, int row_width, float* out, const int* cu,
-                      const int* seq_slots, float* S, int num_seqs, int heads, int P, int N, int groups,
+                      const int* seq_slots, float* S, int num_seqs, int tokens, int heads, int P, int N, int groups,
                       hipStream_t stream) {
-    dim3 grid(num_seqs, heads);
-    const int need = P > N ? P : N;
-    dim3 block(((need + 63) / 64) * 64);
-#define RL_SSM(NMAX)                                                                                             \
-    hipLaunchKernelGGL((recurrent::ssm_scan_kernel<T, NMAX>), grid, block, 0, stream, mixed, dt_raw, dt_bias, a_log, \
-                       skip, packed, row_width, out, cu, seq_slots, S, heads, P, N, groups)
-    if (N <= 16)
-        RL_SSM(16);
-    else if (N <= 32)
-        RL_SSM(32);
-    else if (N <= 64)
-        RL_SSM(64);
-    else if (N <= 128)
-        RL_SSM(128);
+    dim3 grid(num_seqs, heads, (P + 15) / 16);
+#define RL_SSM(RPL)                                                                                           \
+    hipLaunchKernelGGL((recurrent::ssm_scan_kernel<T, RPL>), grid, dim3(recurrent::SCAN_THREADS), 0, stream, mixed, \
+                       dt_raw, dt_bias, a_log, skip, packed, row_width, out, cu, seq_slots, S, heads, P, N, groups)
+    const int rows = (N + 15) / 16;
+    if (rows <= 1)
+        RL_SSM(1);
+    else if (rows <= 2)
+        RL_SSM(2);
+    else if (rows <= 4)
+        RL_SSM(4);
+    else if (rows <= 8)
+        RL_SSM(8);
     else
-        RL_SSM(256);
+        RL_SSM(16);
 #undef RL_SSM
     return rl_launch_status();
 }
 
 extern "C" int rl_ssm_scan(const float* mixed, const float* dt_raw, const float* dt_bias, const float* a_log,
-                           const float* skip, const void* packed, int row_width, float* out, const int* cu,
-                           const int* seq_slots, float* S, int num_seqs, int heads, int P, int N, int groups,
-                           int act_type, hipStream_t stream) {
-    if (num_seqs <= 0) return RL_OK;
+                           const float* skip, const void* packed, int row_width, float* out,
+                           const int* cu, const int* seq_slots, float* S, int num_seqs, int tokens, int heads, int P,
+                           int N, int groups, int act_type, hipStream_t stream) {
+    if (num_seqs <= 0 || tokens <= 0) return RL_OK;
     if (heads < 1 || heads > 65535 || groups < 1 || heads % groups || P < 1 || P > 256 || N < 1 || N > 256 ||
-        row_width < heads * P)
+        row_width < heads * P || num_seqs > 65535)
         return RL_ERR_ARG;
     if (act_type == RL_F32)
         return launch_ssm<float>(mixed, dt_raw, dt_bias, a_log, skip, (const float*)packed, row_width, out, cu,
-                                 seq_slots, S, num_seqs, heads, P, N, groups, stream);
+                                 seq_slots, S, num_seqs, tokens, heads, P, N, groups, stream);
     if (act_type == RL_BF16)
-        return launch_ssm<bf16_t>(mixed, dt_raw, dt_bias, a_log, skip, (const bf16_t*)packed, row_width, out, cu,
-                                  seq_slots, S, num_seqs, heads, P, N, groups, stream);
+        return launch_ssm<bf16_t>(mixed, dt_raw, dt_bias, a_log, skip, (const bf16_t*)packed, row_width, out,
+                                  cu, seq_slots, S, num_seqs, tokens, heads, P, N, groups, stream);
     return RL_ERR_ARG;
 }
 

@@ -2052,9 +2052,9 @@ def wkv(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, deca
         S: torch.Tensor, heads: int, d: int, eps: float) -> None:
     """The time-mixing recurrence between its projections and its output projection.  ``r, k, v,
     g [T, heads * d]``; ``decay_pre`` float32: the decay of a key channel is ``exp(-exp(decay_pre +
-    decay_bias))``; ``bonus [heads, d]`` weighs the current token's own key.  Per head, with the
-    state ``S [slots, heads, d, d]`` (float32, key channel first) read at the rows
-    ``ctx.seq_slots`` and left as it is after each request's last token::
+    decay_bias))``; ``bonus [heads, d]`` weighs the current token's own key.  Per head, with the state ``S [slots, heads, d, d]`` (float32, kept
+    value channel first: ``S[.., j, i]`` belongs to key channel ``i`` and value channel ``j``) read at
+    the rows ``ctx.seq_slots`` and left as it is after each request's last token::
 
         o = (S + diag(bonus) k v^T)^T r        S <- diag(decay) S + k v^T
 
@@ -2071,10 +2071,11 @@ def wkv(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, deca
     _need(norm_weight, "head norm weight", torch.float32, (inner,))
     _need(S, "state", torch.float32, (None, heads, d, d))
     _step_requests(ctx, tokens, S.shape[0])
+    raw = torch.empty((tokens, inner), dtype=torch.float32, device=r.device)  # the heads' outputs before their norm
     _ok(
         recurrent_lib().rl_wkv_scan(_p(r), _p(k), _p(v), _p(g), _p(decay_pre), _p(decay_bias), _p(bonus),
-                                    _p(norm_weight), _p(out), _p(ctx.cu_seqlens), _p(ctx.seq_slots), _p(S),
-                                    ctx.num_seqs, heads, d, ctypes.c_float(eps), _tag(r.dtype), _stream()),
+                                    _p(norm_weight), _p(out), _p(raw), _p(ctx.cu_seqlens), _p(ctx.seq_slots), _p(S),
+                                    ctx.num_seqs, tokens, heads, d, ctypes.c_float(eps), _tag(r.dtype), _stream()),
         "rl_wkv_scan",
     )
 
@@ -2110,8 +2111,8 @@ def state_space_scan(mixed: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.T
     """The state-space recurrence.  ``mixed [T, heads * p + 2 * groups * n]`` float32: ``x``, ``B``
     and ``C`` behind their convolution; ``dt_raw [T, heads]`` float32.  Per head (which reads group
     ``head // (heads / groups)``), with ``dt = softplus(dt_raw + dt_bias)`` and the state ``S [slots,
-    heads, n, p]`` (float32) read at the rows ``ctx.seq_slots`` and left after each request's
-    last token::
+    heads, p, n]`` (float32, the head's channel first) read at the rows ``ctx.seq_slots`` and left
+    after each request's last token::
 
         S <- exp(-exp(decay_log) dt) S + dt B x^T        y = S^T C + skip x
 
@@ -2128,12 +2129,12 @@ def state_space_scan(mixed: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.T
     if packed.shape[1] < inner:
         raise KernelError(f"packed rows of {packed.shape[1]} hold no gate of {inner} channels")
     _need(out, "out", torch.float32, (tokens, inner))
-    _need(S, "state", torch.float32, (None, heads, n, p))
+    _need(S, "state", torch.float32, (None, heads, p, n))
     _step_requests(ctx, tokens, S.shape[0])
     _ok(
         recurrent_lib().rl_ssm_scan(_p(mixed), _p(dt_raw), _p(dt_bias), _p(decay_log), _p(skip), _p(packed),
-                                    packed.shape[1], _p(out), _p(ctx.cu_seqlens), _p(ctx.seq_slots), _p(S),
-                                    ctx.num_seqs, heads, p, n, groups, _tag(packed.dtype), _stream()),
+                                    packed.shape[1], _p(out), _p(ctx.cu_seqlens), _p(ctx.seq_slots),
+                                    _p(S), ctx.num_seqs, tokens, heads, p, n, groups, _tag(packed.dtype), _stream()),
         "rl_ssm_scan",
     )
 

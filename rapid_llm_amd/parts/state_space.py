@@ -107,7 +107,7 @@ class StateSpace(Mixer):
             "state",
             states=(
                 StateSpec("conv", (max(self.taps - 1, 1), self.channels), "float32"),
-                StateSpec("S", (self.heads, self.n, self.p), "float32"),
+                StateSpec("S", (self.heads, self.p, self.n), "float32"),  # a channel's states side by side
             ),
         )
 

@@ -105,7 +105,7 @@ class WKV(Mixer):
             "state",
             states=(
                 StateSpec("shift", (self.hidden_size,), "float32"),
-                StateSpec("S", (self.heads, self.d, self.d), "float32"),
+                StateSpec("S", (self.heads, self.d, self.d), "float32"),  # [value channel, key channel]
             ),
         )
 

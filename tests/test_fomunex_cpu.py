@@ -121,7 +121,7 @@ def test_cache_needs_one_state_for_every_place():
     assert [n.kind for n in needs] == ["paged", "state", "state", "paged", "state", "state"]
     assert needs[0].window == needs[3].window == 19 and needs[3].share_with is None
     assert {s.name: s.shape for s in needs[1].states} == {"shift": (96,), "S": (3, 16, 16)}
-    assert {s.name: s.shape for s in needs[2].states} == {"conv": (2, 64 + 2 * 2 * 24), "S": (4, 24, 16)}
+    assert {s.name: s.shape for s in needs[2].states} == {"conv": (2, 64 + 2 * 2 * 24), "S": (4, 16, 24)}
     assert all(s.dtype == "float32" for n in needs for s in n.states)
 
 

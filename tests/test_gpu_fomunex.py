@@ -211,7 +211,7 @@ def test_convolution_and_state_space_scan_continue_from_the_slot(dtype, heads, P
             packed[:, inner : inner + channels].double(), dt_raw.double(), packed[:, :inner].double(), conv.double(),
             conv_b.double(), dt_bias.double(), a_log.double(), skip.double(), heads, P, N, groups)
     conv_state = torch.zeros((3, max(taps - 1, 1), channels), device=DEV)
-    S = torch.zeros((3, heads, N, P), device=DEV)
+    S = torch.zeros((3, heads, P, N), device=DEV)
     slot = {"a": 2, "b": 0}
     cuts = {"a": _cuts(41, (1, 1, 2, 1, 3, 9, 2)), "b": _cuts(18, (2, 1, 1, 1, 7))}
     got = {rid: ([], []) for rid in lengths}
