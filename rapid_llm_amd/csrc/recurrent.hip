@@ -140,6 +140,20 @@ __device__ inline float row16_sum(float v) {
     v = ror_add<0x121>(v);  // row_ror:1
     return v;
 }
+// the same sums for N values at once, one rotation of all of them after the other: a value's four
+// additions depend on each other, those of different values do not, and a wave that runs alone on
+// its SIMD has nothing else to put between dependent instructions
+template <int N>
+__device__ inline void row16_sums(float (&v)[N]) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] = ror_add<0x128>(v[i]);
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] = ror_add<0x124>(v[i]);
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] = ror_add<0x122>(v[i]);
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] = ror_add<0x121>(v[i]);
+}
 
 constexpr int SCAN_TOKENS = 16;   // tokens staged at a time
 constexpr int SCAN_THREADS = 256;  // 4 waves: 16 columns
@@ -161,7 +175,7 @@ __device__ inline void wkv_row(float r, float k, float w, float u, float vj, flo
 __device__ inline float wkv_decay(float pre, float bias) { return expf(-expf(pre + bias)); }
 
 template <typename T, int RPL>
-__global__ __launch_bounds__(SCAN_THREADS) void wkv_scan_kernel(
+__global__ __launch_bounds__(SCAN_THREADS) __attribute__((amdgpu_waves_per_eu(1, 2))) void wkv_scan_kernel(
     const T* __restrict__ r, const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ decay_pre,
     const float* __restrict__ decay_bias, const float* __restrict__ bonus, float* __restrict__ raw,
     const int* __restrict__ cu,
@@ -219,22 +233,33 @@ __global__ __launch_bounds__(SCAN_THREADS) void wkv_scan_kernel(
         __syncthreads();
         if (tb + SCAN_TOKENS < t1) fetch(tb + SCAN_TOKENS);
         const int nt = min(SCAN_TOKENS, t1 - tb);
-        auto token = [&](int tt) {
+        auto token = [&](int tt) -> float {  // this lane's rows' share of the token's output
             const float vj = sv[tt][col];
             float o = 0.f;
 #pragma unroll
             for (int ii = 0; ii < RPL; ++ii)
                 wkv_row(sr[tt][c * RPL + ii], sk[tt][c * RPL + ii], sw[tt][c * RPL + ii], u[ii], vj, state[ii], o);
-            o = row16_sum(o);
-            if (c == 0 && live) raw[(size_t)(tb + tt) * inner + h * d + j] = o;
+            return o;
         };
+        float* dst = raw + (size_t)tb * inner + h * d + j;
         if (nt == SCAN_TOKENS) {
-            // a whole block, unrolled: the reads of later tokens stand in front of the sums of
-            // earlier ones, and only the state's own chain orders the tokens
+            // a whole block, unrolled and without a branch between its tokens: the reads of later
+            // tokens stand in front of the sums of earlier ones, the lane folds of neighbouring
+            // tokens interleave, and only the state's own chain orders the tokens; the block's
+            // outputs are stored behind it
+            float os[SCAN_TOKENS];
 #pragma unroll
-            for (int tt = 0; tt < SCAN_TOKENS; ++tt) token(tt);
+            for (int tt = 0; tt < SCAN_TOKENS; ++tt) os[tt] = token(tt);
+            row16_sums(os);
+            if (c == 0 && live) {
+#pragma unroll
+                for (int tt = 0; tt < SCAN_TOKENS; ++tt) dst[(size_t)tt * inner] = os[tt];
+            }
         } else {
-            for (int tt = 0; tt < nt; ++tt) token(tt);
+            for (int tt = 0; tt < nt; ++tt) {
+                const float o = row16_sum(token(tt));
+                if (c == 0 && live) dst[(size_t)tt * inner] = o;
+            }
         }
     }
     if (live) {
@@ -365,7 +390,7 @@ __device__ inline void ssm_row(float a, float B, float C, float dx, float& state
 __device__ inline float ssm_out(float y, float D, float x, float z) { return fmaf(D, x, y) * silu(z); }
 
 template <typename T, int RPL>
-__global__ __launch_bounds__(SCAN_THREADS) void ssm_scan_kernel(
+__global__ __launch_bounds__(SCAN_THREADS) __attribute__((amdgpu_waves_per_eu(1, 2))) void ssm_scan_kernel(
     const float* __restrict__ mixed, const float* __restrict__ dt_raw, const float* __restrict__ dt_bias,
     const float* __restrict__ a_log, const float* __restrict__ skip, const T* __restrict__ packed, int row_width, float* __restrict__ out, const int* __restrict__ cu,
     const int* __restrict__ seq_slots, float* __restrict__ S, int heads, int P, int N, int groups) {
@@ -430,21 +455,33 @@ __global__ __launch_bounds__(SCAN_THREADS) void ssm_scan_kernel(
         __syncthreads();
         if (tb + SCAN_TOKENS < t1) fetch(tb + SCAN_TOKENS);
         const int nt = min(SCAN_TOKENS, t1 - tb);
-        auto token = [&](int tt) {
+        auto token = [&](int tt) -> float {
             const float x = sx[tt][col], a = sa[tt];
             const float dx = sdt[tt] * x;
             float y = 0.f;
 #pragma unroll
             for (int ii = 0; ii < RPL; ++ii)
                 ssm_row(a, sB[tt][c * RPL + ii], sC[tt][c * RPL + ii], dx, state[ii], y);
-            y = row16_sum(y);
-            if (c == 0 && live) out[(size_t)(tb + tt) * inner + h * P + p] = ssm_out(y, D, x, sz[tt][col]);
+            return y;  // this lane's rows' share
         };
+        float* dst = out + (size_t)tb * inner + h * P + p;
         if (nt == SCAN_TOKENS) {
+            // a whole block without a branch between its tokens; its outputs are finished and
+            // stored behind it
+            float ys[SCAN_TOKENS];
 #pragma unroll
-            for (int tt = 0; tt < SCAN_TOKENS; ++tt) token(tt);
+            for (int tt = 0; tt < SCAN_TOKENS; ++tt) ys[tt] = token(tt);
+            row16_sums(ys);
+            if (c == 0 && live) {
+#pragma unroll
+                for (int tt = 0; tt < SCAN_TOKENS; ++tt)
+                    dst[(size_t)tt * inner] = ssm_out(ys[tt], D, sx[tt][col], sz[tt][col]);
+            }
         } else {
-            for (int tt = 0; tt < nt; ++tt) token(tt);
+            for (int tt = 0; tt < nt; ++tt) {
+                const float y = row16_sum(token(tt));
+                if (c == 0 && live) dst[(size_t)tt * inner] = ssm_out(y, D, sx[tt][col], sz[tt][col]);
+            }
         }
     }
     if (live) {
