@@ -130,7 +130,7 @@ __global__ __launch_bounds__(256) void shift_state_kernel(const T* __restrict__ 
 // --------------------------------------------------------------------------- //
 template <int CTRL>
 __device__ inline float ror_add(float v) {
-    const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false);
+    const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true);
     return v + __int_as_float(moved);
 }
 __device__ inline float row16_sum(float v) {
@@ -156,7 +156,9 @@ __device__ inline void row16_sums(float (&v)[N]) {
 }
 
 constexpr int SCAN_TOKENS = 16;   // tokens staged at a time
-constexpr int SCAN_THREADS = 256;  // 4 waves: 16 columns
+constexpr int SCAN_WAVES = 4;                      // waves of a workgroup
+constexpr int SCAN_THREADS = 64 * SCAN_WAVES;
+constexpr int SCAN_COLS = 4 * SCAN_WAVES;          // columns of a workgroup: 4 a wave
 
 // --------------------------------------------------------------------------- //
 // The time-mixing scan.  Per head, state S[key channel i][value channel j], kept as [j][i].  For a
@@ -187,11 +189,11 @@ __global__ __launch_bounds__(SCAN_THREADS) __attribute__((amdgpu_waves_per_eu(1,
     const int inner = heads * d;
     const int lane = threadIdx.x & (RL_WAVE - 1), wave = threadIdx.x / RL_WAVE;
     const int c = lane & 15;                                  // which share of the rows
-    const int col = wave * 4 + (lane >> 4);                   // column of the workgroup's 16
-    const int j = blockIdx.z * 16 + col;
+    const int col = wave * 4 + (lane >> 4);                   // column of the workgroup
+    const int j = blockIdx.z * SCAN_COLS + col;
     const bool live = j < d;
     __shared__ __attribute__((aligned(16))) float sr[SCAN_TOKENS][DP], sk[SCAN_TOKENS][DP], sw[SCAN_TOKENS][DP];
-    __shared__ float sv[SCAN_TOKENS][16];
+    __shared__ float sv[SCAN_TOKENS][SCAN_COLS];
     float* Sp = S + (((size_t)seq_slots[s] * heads + h) * d + (live ? j : 0)) * d;
     float state[RPL], u[RPL];
 #pragma unroll
@@ -200,8 +202,18 @@ __global__ __launch_bounds__(SCAN_THREADS) __attribute__((amdgpu_waves_per_eu(1,
         state[ii] = (live && i < d) ? Sp[i] : 0.f;
         u[ii] = i < d ? bonus[h * d + i] : 0.f;
     }
-    // a block of tokens from memory into registers: element e of the block's [token][row] arrays
-    float pr[PER_THREAD], pk[PER_THREAD], pw[PER_THREAD], pv = 0.f;
+    // A block of tokens from memory into registers, as it lies there: element e of the block's
+    // [token][row] arrays.  Nothing is computed from what was asked for until the block is staged
+    // (a conversion or an exponential here would wait for the loads where they are issued, and
+    // the block before would be computed behind that wait instead of during it).
+    T pr[PER_THREAD], pk[PER_THREAD], pv;
+    float pw[PER_THREAD], pb[PER_THREAD];
+#pragma unroll
+    for (int e = 0; e < PER_THREAD; ++e) {
+        const int i = (e * SCAN_THREADS + threadIdx.x) % DP;
+        pb[e] = i < d ? decay_bias[h * d + i] : 0.f;
+    }
+    const T zero = from_float<T>(0.f);
     auto fetch = [&](int tb) {
 #pragma unroll
         for (int e = 0; e < PER_THREAD; ++e) {
@@ -209,22 +221,23 @@ __global__ __launch_bounds__(SCAN_THREADS) __attribute__((amdgpu_waves_per_eu(1,
             const int tt = idx / DP, i = idx % DP;
             const bool ok = tb + tt < t1 && i < d;
             const size_t at = (size_t)(tb + tt) * inner + h * d + i;
-            pr[e] = ok ? to_float(r[at]) : 0.f;
-            pk[e] = ok ? to_float(k[at]) : 0.f;
-            pw[e] = ok ? wkv_decay(decay_pre[at], decay_bias[h * d + i]) : 0.f;
+            pr[e] = ok ? r[at] : zero;
+            pk[e] = ok ? k[at] : zero;
+            pw[e] = ok ? decay_pre[at] : INFINITY;  // a decay of exactly 0
         }
-        const int tt = threadIdx.x / 16, jj = blockIdx.z * 16 + (threadIdx.x & 15);
-        pv = (tb + tt < t1 && jj < d) ? to_float(v[(size_t)(tb + tt) * inner + h * d + jj]) : 0.f;
+        // (threads beyond tokens x columns, where a workgroup has more, carry nothing)
+        const int tt = threadIdx.x / SCAN_COLS, jj = blockIdx.z * SCAN_COLS + threadIdx.x % SCAN_COLS;
+        pv = (tt < SCAN_TOKENS && tb + tt < t1 && jj < d) ? v[(size_t)(tb + tt) * inner + h * d + jj] : zero;
     };
     auto stage = [&]() {
 #pragma unroll
         for (int e = 0; e < PER_THREAD; ++e) {
             const int idx = e * SCAN_THREADS + threadIdx.x;
-            (&sr[0][0])[idx] = pr[e];
-            (&sk[0][0])[idx] = pk[e];
-            (&sw[0][0])[idx] = pw[e];
+            (&sr[0][0])[idx] = to_float(pr[e]);
+            (&sk[0][0])[idx] = to_float(pk[e]);
+            (&sw[0][0])[idx] = wkv_decay(pw[e], pb[e]);
         }
-        (&sv[0][0])[threadIdx.x] = pv;
+        if (threadIdx.x < SCAN_TOKENS * SCAN_COLS) (&sv[0][0])[threadIdx.x] = to_float(pv);
     };
     fetch(t0);
     for (int tb = t0; tb < t1; tb += SCAN_TOKENS) {
@@ -251,10 +264,11 @@ __global__ __launch_bounds__(SCAN_THREADS) __attribute__((amdgpu_waves_per_eu(1,
 #pragma unroll
             for (int tt = 0; tt < SCAN_TOKENS; ++tt) os[tt] = token(tt);
             row16_sums(os);
-            if (c == 0 && live) {
+            // every lane of a column holds all sixteen sums: lane c stores token c's
+            float mine = os[0];
 #pragma unroll
-                for (int tt = 0; tt < SCAN_TOKENS; ++tt) dst[(size_t)tt * inner] = os[tt];
-            }
+            for (int tt = 1; tt < SCAN_TOKENS; ++tt) mine = c == tt ? os[tt] : mine;
+            if (live) dst[(size_t)c * inner] = mine;
         } else {
             for (int tt = 0; tt < nt; ++tt) {
                 const float o = row16_sum(token(tt));
@@ -404,16 +418,20 @@ __global__ __launch_bounds__(SCAN_THREADS) __attribute__((amdgpu_waves_per_eu(1,
     const int lane = threadIdx.x & (RL_WAVE - 1), wave = threadIdx.x / RL_WAVE;
     const int c = lane & 15;
     const int col = wave * 4 + (lane >> 4);
-    const int p = blockIdx.z * 16 + col;
+    const int p = blockIdx.z * SCAN_COLS + col;
     const bool live = p < P;
     __shared__ __attribute__((aligned(16))) float sB[SCAN_TOKENS][NP], sC[SCAN_TOKENS][NP];
-    __shared__ float sx[SCAN_TOKENS][16], sz[SCAN_TOKENS][16], sdt[SCAN_TOKENS], sa[SCAN_TOKENS];
+    __shared__ float sx[SCAN_TOKENS][SCAN_COLS], sz[SCAN_TOKENS][SCAN_COLS], sdt[SCAN_TOKENS], sa[SCAN_TOKENS];
     float* Sp = S + (((size_t)seq_slots[s] * heads + h) * P + (live ? p : 0)) * N;
     float state[RPL];
 #pragma unroll
     for (int ii = 0; ii < RPL; ++ii) state[ii] = (live && c * RPL + ii < N) ? Sp[c * RPL + ii] : 0.f;
     const float D = skip[h];
-    float pB[PER_THREAD], pC[PER_THREAD], px = 0.f, pz = 0.f, pd = 0.f;
+    // a block of tokens from memory into registers as it lies there; step sizes and decays are
+    // formed when the block is staged, not where its loads are issued
+    float pB[PER_THREAD], pC[PER_THREAD], px = 0.f, pd = 0.f;
+    T pz = from_float<T>(0.f);
+    const float step_bias = dt_bias[h], rate_log = a_log[h];
     auto fetch = [&](int tb) {
 #pragma unroll
         for (int e = 0; e < PER_THREAD; ++e) {
@@ -424,17 +442,13 @@ __global__ __launch_bounds__(SCAN_THREADS) __attribute__((amdgpu_waves_per_eu(1,
             pB[e] = ok ? row[0] : 0.f;
             pC[e] = ok ? row[groups * N] : 0.f;
         }
-        const int tt = threadIdx.x / 16, pp = blockIdx.z * 16 + (threadIdx.x & 15);
-        const bool ok = tb + tt < t1 && pp < P;
+        const int tt = threadIdx.x / SCAN_COLS, pp = blockIdx.z * SCAN_COLS + threadIdx.x % SCAN_COLS;
+        const bool ok = tt < SCAN_TOKENS && tb + tt < t1 && pp < P;
         px = ok ? mixed[(size_t)(tb + tt) * channels + h * P + pp] : 0.f;
-        pz = ok ? to_float(packed[(size_t)(tb + tt) * row_width + h * P + pp]) : 0.f;
+        pz = ok ? packed[(size_t)(tb + tt) * row_width + h * P + pp] : from_float<T>(0.f);
         // threads 0..15 carry the step sizes, threads 16..31 the decays of the block's tokens
-        const int which = threadIdx.x / 16, tk = threadIdx.x & 15;
-        pd = 0.f;
-        if (which < 2 && tb + tk < t1) {
-            const float dt = ssm_step_size(dt_raw[(size_t)(tb + tk) * heads + h], dt_bias[h]);
-            pd = which == 0 ? dt : ssm_decay(a_log[h], dt);
-        }
+        const int tk = threadIdx.x & 15;
+        pd = (threadIdx.x < 32 && tb + tk < t1) ? dt_raw[(size_t)(tb + tk) * heads + h] : 0.f;
     };
     auto stage = [&]() {
 #pragma unroll
@@ -443,10 +457,15 @@ __global__ __launch_bounds__(SCAN_THREADS) __attribute__((amdgpu_waves_per_eu(1,
             (&sB[0][0])[idx] = pB[e];
             (&sC[0][0])[idx] = pC[e];
         }
-        (&sx[0][0])[threadIdx.x] = px;
-        (&sz[0][0])[threadIdx.x] = pz;
-        if (threadIdx.x < 16) sdt[threadIdx.x] = pd;
-        else if (threadIdx.x < 32) sa[threadIdx.x - 16] = pd;
+        if (threadIdx.x < SCAN_TOKENS * SCAN_COLS) {
+            (&sx[0][0])[threadIdx.x] = px;
+            (&sz[0][0])[threadIdx.x] = to_float(pz);
+        }
+        if (threadIdx.x < 32) {
+            const float dt = ssm_step_size(pd, step_bias);
+            if (threadIdx.x < 16) sdt[threadIdx.x] = dt;
+            else sa[threadIdx.x - 16] = ssm_decay(rate_log, dt);
+        }
     };
     fetch(t0);
     for (int tb = t0; tb < t1; tb += SCAN_TOKENS) {
@@ -466,17 +485,17 @@ __global__ __launch_bounds__(SCAN_THREADS) __attribute__((amdgpu_waves_per_eu(1,
         };
         float* dst = out + (size_t)tb * inner + h * P + p;
         if (nt == SCAN_TOKENS) {
-            // a whole block without a branch between its tokens; its outputs are finished and
-            // stored behind it
+            // a whole block without a branch between its tokens
             float ys[SCAN_TOKENS];
 #pragma unroll
             for (int tt = 0; tt < SCAN_TOKENS; ++tt) ys[tt] = token(tt);
             row16_sums(ys);
-            if (c == 0 && live) {
+            // every lane of a column holds all sixteen sums: lane c finishes and stores token c's
+            // (skip term, gate with its exponential and division: once a lane, not once a token)
+            float mine = ys[0];
 #pragma unroll
-                for (int tt = 0; tt < SCAN_TOKENS; ++tt)
-                    dst[(size_t)tt * inner] = ssm_out(ys[tt], D, sx[tt][col], sz[tt][col]);
-            }
+            for (int tt = 1; tt < SCAN_TOKENS; ++tt) mine = c == tt ? ys[tt] : mine;
+            if (live) dst[(size_t)c * inner] = ssm_out(mine, D, sx[c][col], sz[c][col]);
         } else {
             for (int tt = 0; tt < nt; ++tt) {
                 const float y = row16_sum(token(tt));
@@ -544,7 +563,7 @@ static int launch_wkv(const T* r, const T* k, const T* v, const T* g, const floa
                       const float* bonus, const float* norm_w, T* out, float* raw, const int* cu,
                       const int* seq_slots, float* S, int num_seqs, int tokens, int heads, int d, float eps,
                       hipStream_t stream) {
-    dim3 grid(num_seqs, heads, (d + 15) / 16);
+    dim3 grid(num_seqs, heads, (d + recurrent::SCAN_COLS - 1) / recurrent::SCAN_COLS);
 #define RL_WKV(RPL)                                                                                              \
     hipLaunchKernelGGL((recurrent::wkv_scan_kernel<T, RPL>), grid, dim3(recurrent::SCAN_THREADS), 0, stream, r, k, v, \
                        decay, decay_bias, bonus, raw, cu, seq_slots, S, heads, d)
@@ -620,7 +639,7 @@ static int launch_ssm(const float* mixed, const float* dt_raw, const float* dt_b
                       const float* skip, const T* packed, int row_width, float* out, const int* cu,
                       const int* seq_slots, float* S, int num_seqs, int tokens, int heads, int P, int N, int groups,
                       hipStream_t stream) {
-    dim3 grid(num_seqs, heads, (P + 15) / 16);
+    dim3 grid(num_seqs, heads, (P + recurrent::SCAN_COLS - 1) / recurrent::SCAN_COLS);
 #define RL_SSM(RPL)                                                                                           \
     hipLaunchKernelGGL((recurrent::ssm_scan_kernel<T, RPL>), grid, dim3(recurrent::SCAN_THREADS), 0, stream, mixed, \
                        dt_raw, dt_bias, a_log, skip, packed, row_width, out, cu, seq_slots, S, heads, P, N, groups)
