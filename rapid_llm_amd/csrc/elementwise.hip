@@ -719,25 +719,21 @@ extern "C" int rl_unary_act(const void* x, void* out, int tokens, int cols, int 
 __device__ inline void route_row(float* __restrict__ row, float* __restrict__ dst, int experts, int top, float scale,
                                  int sigmoid = 0) {
     if (sigmoid) {
-        // the largest logits are the largest scores; a chosen one is marked by a NaN-free trick:
-        // its score, a number in (0, 1), is stored negated
-        for (int e = 0; e < experts; ++e) row[e] = 1.f / (1.f + expf(-row[e]));
+        // The largest scores are the largest logits, and the logits are what is compared: two
+        // scores that round to the same float32 (both 1 beyond a logit of 17) still differ there.
+        // dst (not row: the router kernel's logits lie in LDS) holds 0 until an expert is chosen.
+        for (int e = 0; e < experts; ++e) dst[e] = 0.f;
         for (int k = 0; k < top; ++k) {
             int best = -1;
-            float best_s = -1.f;
+            float best_z = -INFINITY;
             for (int e = 0; e < experts; ++e) {
-                const float p = row[e];
-                if (!signbit(p) && p > best_s) {
-                    best_s = p;
+                if (dst[e] == 0.f && row[e] > best_z) {
+                    best_z = row[e];
                     best = e;
                 }
             }
             if (best < 0) break;
-            row[best] = -best_s;  // -0.f for a score that underflowed: still marked by its sign
-        }
-        for (int e = 0; e < experts; ++e) {
-            const float p = row[e];
-            dst[e] = signbit(p) ? -p * scale : 0.f;
+            dst[best] = scale / (1.f + expf(-best_z));
         }
         return;
     }

@@ -285,6 +285,18 @@ def test_router_with_sigmoid_scores_taken_as_they_are(experts, top):
                                rtol=1e-4, atol=1e-4)
 
 
+def test_router_chooses_among_scores_that_round_to_one():
+    """Logits beyond 17 all have the float32 score 1; the larger logit is still the larger score."""
+    ops = _ops()
+    h = torch.randn(64, 32)
+    w = torch.randn(8, 32) * 6.0
+    z = h.double() @ w.double().T
+    assert int((z > 17).sum(1).max()) >= 2  # the case is there
+    got = ops.router(h.to(DEV), w.to(DEV), 1, 1.0, None, "sigmoid").cpu()
+    assert torch.equal(got.argmax(1), z.argmax(1))
+    assert int((got > 0).sum()) == 64
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("experts,ff,limit", [(5, 27, 1.5), (6, 24, 2.0), (1, 16, 0.5)])
 def test_an_experts_weight_scales_what_it_reads(dtype, experts, ff, limit):
