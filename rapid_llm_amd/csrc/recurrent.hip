@@ -310,7 +310,7 @@ __global__ __launch_bounds__(256) void wkv_finish_kernel(const float* __restrict
 // seen, oldest first; zeros when the request begins).  A second launch then shifts the state; in a
 // step of single tokens (`single`) the thread of a channel shifts its request's rows itself.
 // --------------------------------------------------------------------------- //
-#define RL_CONV_MAX_TAPS 8
+#define RL_CONV_MAX_TAPS 16
 
 constexpr int CONV_TOKENS = 8;  // consecutive tokens of the flat batch a workgroup takes in a step with portions
 

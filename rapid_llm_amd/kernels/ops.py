@@ -2013,7 +2013,7 @@ def mlstm(
 WKV_MAX_HEAD_DIM = 256  # a thread keeps one column of a head's state in registers
 SSM_MAX_STATE = 256
 SSM_MAX_HEAD_DIM = 256
-CONV_MAX_TAPS = 8
+CONV_MAX_TAPS = 16
 
 
 def _step_requests(ctx, tokens: int, slots: int) -> None:

@@ -189,7 +189,7 @@ def _state_space_oracle(xbc, dt_raw, z, conv, conv_b, dt_bias, a_log, skip, head
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("heads,P,N,groups,taps", [(4, 16, 24, 2, 3), (6, 10, 12, 3, 2), (2, 64, 64, 1, 8), (1, 16, 1, 1, 1),
-                                                   (2, 32, 130, 2, 4), (3, 200, 8, 1, 4)])
+                                                   (2, 32, 130, 2, 4), (3, 200, 8, 1, 4), (2, 16, 16, 1, 13)])
 def test_convolution_and_state_space_scan_continue_from_the_slot(dtype, heads, P, N, groups, taps):
     """Portions shorter than the convolution's reach (one, two and three tokens in a row), so that
     the kept inputs are shifted and not replaced; two requests in shared steps."""
