@@ -155,6 +155,45 @@ __device__ inline void row16_sums(float (&v)[N]) {
     for (int i = 0; i < N; ++i) v[i] = ror_add<0x121>(v[i]);
 }
 
+// A lane's RPL consecutive state rows from or to memory: sixteen bytes at a time where the rows
+// of a column are a multiple of four (a group of four is then wholly inside the column or wholly
+// beyond it), else one by one.
+template <int RPL>
+__device__ inline void state_rows_load(const float* __restrict__ column, int first, int rows, bool live,
+                                       float (&state)[RPL]) {
+    if constexpr (RPL % 4 == 0) {
+        if (rows % 4 == 0) {
+#pragma unroll
+            for (int q = 0; q < RPL; q += 4) {
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (live && first + q < rows) v = *reinterpret_cast<const float4*>(column + first + q);
+                state[q] = v.x; state[q + 1] = v.y; state[q + 2] = v.z; state[q + 3] = v.w;
+            }
+            return;
+        }
+    }
+#pragma unroll
+    for (int ii = 0; ii < RPL; ++ii) state[ii] = (live && first + ii < rows) ? column[first + ii] : 0.f;
+}
+template <int RPL>
+__device__ inline void state_rows_store(float* __restrict__ column, int first, int rows, bool live,
+                                        const float (&state)[RPL]) {
+    if (!live) return;
+    if constexpr (RPL % 4 == 0) {
+        if (rows % 4 == 0) {
+#pragma unroll
+            for (int q = 0; q < RPL; q += 4)
+                if (first + q < rows)
+                    *reinterpret_cast<float4*>(column + first + q) =
+                        make_float4(state[q], state[q + 1], state[q + 2], state[q + 3]);
+            return;
+        }
+    }
+#pragma unroll
+    for (int ii = 0; ii < RPL; ++ii)
+        if (first + ii < rows) column[first + ii] = state[ii];
+}
+
 constexpr int SCAN_TOKENS = 16;   // tokens staged at a time
 constexpr int SCAN_WAVES = 4;                      // waves of a workgroup
 constexpr int SCAN_THREADS = 64 * SCAN_WAVES;
@@ -196,10 +235,10 @@ __global__ __launch_bounds__(SCAN_THREADS) __attribute__((amdgpu_waves_per_eu(1,
     __shared__ float sv[SCAN_TOKENS][SCAN_COLS];
     float* Sp = S + (((size_t)seq_slots[s] * heads + h) * d + (live ? j : 0)) * d;
     float state[RPL], u[RPL];
+    state_rows_load<RPL>(Sp, c * RPL, d, live, state);
 #pragma unroll
     for (int ii = 0; ii < RPL; ++ii) {
         const int i = c * RPL + ii;
-        state[ii] = (live && i < d) ? Sp[i] : 0.f;
         u[ii] = i < d ? bonus[h * d + i] : 0.f;
     }
     // A block of tokens from memory into registers, as it lies there: element e of the block's
@@ -276,11 +315,7 @@ __global__ __launch_bounds__(SCAN_THREADS) __attribute__((amdgpu_waves_per_eu(1,
             }
         }
     }
-    if (live) {
-#pragma unroll
-        for (int ii = 0; ii < RPL; ++ii)
-            if (c * RPL + ii < d) Sp[c * RPL + ii] = state[ii];
-    }
+    state_rows_store<RPL>(Sp, c * RPL, d, live, state);
 }
 
 // out[t, head] = raw / sqrt(mean(raw^2) + eps) * norm_w * silu(g): one wave a (token, head)
@@ -424,8 +459,7 @@ __global__ __launch_bounds__(SCAN_THREADS) __attribute__((amdgpu_waves_per_eu(1,
     __shared__ float sx[SCAN_TOKENS][SCAN_COLS], sz[SCAN_TOKENS][SCAN_COLS], sdt[SCAN_TOKENS], sa[SCAN_TOKENS];
     float* Sp = S + (((size_t)seq_slots[s] * heads + h) * P + (live ? p : 0)) * N;
     float state[RPL];
-#pragma unroll
-    for (int ii = 0; ii < RPL; ++ii) state[ii] = (live && c * RPL + ii < N) ? Sp[c * RPL + ii] : 0.f;
+    state_rows_load<RPL>(Sp, c * RPL, N, live, state);
     const float D = skip[h];
     // a block of tokens from memory into registers as it lies there; step sizes and decays are
     // formed when the block is staged, not where its loads are issued
@@ -503,11 +537,7 @@ __global__ __launch_bounds__(SCAN_THREADS) __attribute__((amdgpu_waves_per_eu(1,
             }
         }
     }
-    if (live) {
-#pragma unroll
-        for (int ii = 0; ii < RPL; ++ii)
-            if (c * RPL + ii < N) Sp[c * RPL + ii] = state[ii];
-    }
+    state_rows_store<RPL>(Sp, c * RPL, N, live, state);
 }
 
 // out[t, part] = y[t, part] / sqrt(mean(y[t, part]^2) + eps) * w, a row in `parts` equal parts
