@@ -244,9 +244,7 @@ class FomunexConfig:
         for i, layer in enumerate(layers):
             if layer.weights_of is None:
                 continue
-            owner = layers[layer.weights_of]
-            if owner.weights_of is not None:
-                raise ConfigError(f"layers[{i}]: layer {layer.weights_of} has no tensors of its own")
+            owner = layers[cls._owner(layers, i)]
             if (owner.type, owner.mixer, owner.mlp) != (layer.type, layer.mixer, layer.mlp):
                 raise ConfigError(f"layers[{i}] uses the tensors of layer {layer.weights_of} but differs from it")
         norm = data.get("norm") or {}
@@ -271,9 +269,20 @@ class FomunexConfig:
             eos_token_ids=eos_ids,
         )
 
+    @staticmethod
+    def _owner(layers, i: int) -> int:
+        """The layer whose tensors layer ``i`` runs: ``weights_of`` followed until a layer that has its own."""
+        seen = set()
+        while layers[i].weights_of is not None:
+            if i in seen:
+                raise ConfigError(f"layers[{i}]: weights_of leads back to the layer itself")
+            seen.add(i)
+            i = layers[i].weights_of
+        return i
+
     def run_order(self) -> tuple[int, ...]:
         """For every place in the run order, the layer whose tensors run there."""
-        return tuple(i if layer.weights_of is None else layer.weights_of for i, layer in enumerate(self.layers))
+        return tuple(self._owner(self.layers, i) for i in range(len(self.layers)))
 
     def to_dict(self) -> dict[str, Any]:
         out: dict[str, Any] = {

@@ -40,6 +40,20 @@ def test_configuration_round_trip_and_run_order(which):
     assert spec.max_position == cfg["max_positions"]
 
 
+def test_a_layer_may_name_a_layer_that_names_another():
+    cfg, _page, _seed = FOMU["A"]
+    chained = copy.deepcopy(cfg)
+    chained["layers"].append(dict(copy.deepcopy(cfg["layers"][3]), weights_of=3))  # 6 -> 3 -> 0
+    chained["layers"].insert(0, dict(copy.deepcopy(cfg["layers"][2]), weights_of=3))  # the owner comes later
+    for layer in chained["layers"][1:]:
+        if layer.get("weights_of") is not None:
+            layer["weights_of"] += 1
+    _entry, typed, spec = _spec(chained)
+    assert typed.run_order() == (3, 1, 2, 3, 1, 2, 6, 1)
+    assert len(spec.layers) == 4 and list(spec.order()) == [2, 0, 1, 2, 0, 1, 3, 0]
+    assert spec.layers[2].checkpoint_prefix == "l3."
+
+
 def test_configuration_refuses_what_the_design_does_not_have():
     from rapid_llm_amd.config.model_config import ConfigError
 
@@ -47,7 +61,7 @@ def test_configuration_refuses_what_the_design_does_not_have():
     for change in (
         lambda c: c["layers"][0].update(type="convolution"),
         lambda c: c["layers"][3].update(weights_of=3),
-        lambda c: c["layers"][3].update(weights_of=4),  # a layer without tensors of its own
+        lambda c: (c["layers"][0].update(weights_of=3)),  # two layers that name each other
         lambda c: c["layers"][3]["mixer"].update(heads=8),  # differs from the layer whose tensors it uses
         lambda c: c["layers"][2]["mixer"].update(groups=3),
         lambda c: c["layers"][2]["mixer"].update(norm_groups=7),
